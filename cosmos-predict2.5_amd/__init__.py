@@ -1,0 +1,13 @@
+"""MI355X-native flash-attention forward + forward-mode JVP for Cosmos-Predict2.5's DiT attention.
+
+The directory name is not a Python identifier; load it with ``__graft_entry__.load_package()``
+(registers it as ``cosmos_predict2_5_amd``).
+"""
+from . import _lib  # noqa: F401
+from .attention import attention as attention_forward
+from .attn_op import HipAttnOp, hip_attention_op
+from .flash_attention_jvp import attention as attention_jvp
+from .flash_attention_jvp import attention_with_lse
+from .ops import fwd_jvp
+
+__all__ = ["attention_jvp", "attention_with_lse", "attention_forward", "HipAttnOp", "hip_attention_op", "fwd_jvp"]

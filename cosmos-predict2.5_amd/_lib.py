@@ -1,0 +1,100 @@
+"""ctypes binding of ``libcosmos_attn_hip.so`` (declarations: ``include/cosmos_attn_hip.h``).
+
+There is no fallback: if the library is missing or its ABI version differs, importing the
+operators raises.  ``import torch`` must happen before the library is loaded so that both use the
+one HIP runtime already in the process (this module imports torch first for that reason).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch  # noqa: F401  (loads the HIP runtime the library binds to)
+
+from .build import LIB_PATH
+
+ABI_VERSION = 1
+DTYPE_BF16, DTYPE_FP16 = 0, 1
+
+ST_OK, ST_BAD_ARG, ST_BAD_SHAPE, ST_BAD_STRIDE, ST_UNSUPPORTED, ST_WORKSPACE, ST_LAUNCH = range(7)
+
+
+class AttnDesc(ctypes.Structure):
+    """Mirror of ``struct cosmos_attn_desc``."""
+
+    _fields_ = [
+        ("abi_version", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("B", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("Lq", ctypes.c_int32),
+        ("Lkv", ctypes.c_int32),
+        ("d_qk", ctypes.c_int32),
+        ("d_v", ctypes.c_int32),
+        ("causal", ctypes.c_int32),
+        ("sm_scale", ctypes.c_float),
+        ("q", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("tq", ctypes.c_void_p),
+        ("tk", ctypes.c_void_p),
+        ("tv", ctypes.c_void_p),
+        ("q_stride", ctypes.c_int64 * 3),
+        ("k_stride", ctypes.c_int64 * 3),
+        ("v_stride", ctypes.c_int64 * 3),
+        ("o", ctypes.c_void_p),
+        ("to", ctypes.c_void_p),
+        ("o_stride", ctypes.c_int64 * 3),
+        ("lse", ctypes.c_void_p),
+        ("key_lens", ctypes.c_void_p),
+    ]
+
+
+EXPORTS = {
+    "cosmos_attn_abi_version": (ctypes.c_int, []),
+    "cosmos_attn_status_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "cosmos_attn_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(AttnDesc)]),
+    "cosmos_attn_fwd_jvp": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "cosmos_attn_pack_kv": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "cosmos_attn_run": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+}
+
+_lib = None
+
+
+def load_library() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: the HIP attention library has not been built "
+            f"(run `python __graft_entry__.py build`). There is no fallback path."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in EXPORTS.items():
+        fn = getattr(lib, name)  # AttributeError if a declared symbol is not exported
+        fn.restype, fn.argtypes = restype, argtypes
+    got = lib.cosmos_attn_abi_version()
+    if got != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {got}, expected {ABI_VERSION}; rebuild the library")
+    _lib = lib
+    return lib
+
+
+def status_string(status: int) -> str:
+    return load_library().cosmos_attn_status_string(status).decode()
+
+
+def raise_for_status(status: int) -> None:
+    """Status code -> the exception type the reference raises for the same condition."""
+    if status == ST_OK:
+        return
+    msg = f"cosmos_attn: {status_string(status)} (status {status})"
+    if status in (ST_BAD_SHAPE, ST_BAD_STRIDE):
+        raise AssertionError(msg)
+    if status == ST_UNSUPPORTED:
+        raise NotImplementedError(msg)
+    if status == ST_BAD_ARG:
+        raise ValueError(msg)
+    raise RuntimeError(msg)

@@ -1,0 +1,50 @@
+"""Drop-in for the reference's forward attention entry used by the DiT blocks.
+
+Reference: cosmos_predict2/_src/predict2/networks/attention.py ``attention(q, k, v, q_lens=None,
+k_lens=None, dropout_p=0.0, softmax_scale=None, q_scale=None, causal=False, deterministic=False,
+dtype=torch.bfloat16) -> out`` (:90-181), tensors ``[B, S, H, D]``, output contiguous ``[B, S, H, D]`` (:180).
+
+Behaviour kept: cast of q,k,v to ``dtype`` (:110-112), ``q_scale`` (:114-115), ``NotImplementedError`` for
+unsupported dtypes (:107-108), ``q_lens`` / ``k_lens`` accepted and ignored (:94-95 -- the reference never
+reads them).  The gfx950 kernels are deterministic (no atomics, fixed reduction order), so
+``deterministic=True`` is honoured instead of raising (:151-154).  fp32 is not built: NotImplementedError.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+
+
+def attention(
+    q,
+    k,
+    v,
+    q_lens=None,
+    k_lens=None,
+    dropout_p=0.0,
+    softmax_scale=None,
+    q_scale=None,
+    causal=False,
+    deterministic=False,
+    dtype=torch.bfloat16,
+):
+    supported_dtypes = [torch.bfloat16, torch.float16]
+    if dtype not in supported_dtypes:
+        raise NotImplementedError(f"{dtype=} is not supported.")
+    if dropout_p != 0.0:
+        raise NotImplementedError("dropout is not supported by the HIP attention kernels")
+    del q_lens, k_lens, deterministic
+
+    q = q.to(dtype)
+    k = k.to(dtype)
+    v = v.to(dtype)
+    if q_scale is not None:
+        q = q * q_scale
+
+    # [B, S, H, D] -> heads-first views (no copy); the kernel writes [B, S, H, D] memory directly
+    o, _, _ = ops.fwd_jvp(
+        q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
+        causal=causal, sm_scale=softmax_scale, out_layout="blhd", need_lse=False,
+    )
+    return o.transpose(1, 2)

@@ -1,0 +1,138 @@
+"""Host side of the HIP attention forward + JVP: argument checks, workspace, launch.
+
+``fwd_jvp`` is the one function that talks to the C ABI.  It takes heads-first views
+``[B, H, L, d]`` (any batch/head/row strides, innermost stride 1), launches on torch's current
+stream, never synchronises, and allocates outputs with ``torch.empty`` like the reference wrapper
+(cosmos_predict2/_src/predict2/utils/flash_attention_jvp_triton.py:451-455).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
+SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)
+REFERENCE_HEAD_DIMS = (16, 32, 64, 128, 256)  # what the reference accepts (…jvp_triton.py:444-445)
+
+
+def _kernel_ready(x: torch.Tensor) -> bool:
+    """True if the view can be handed to the kernel as is: d stride 1, 16-byte rows and base."""
+    return (
+        x.stride(-1) == 1
+        and x.data_ptr() % 16 == 0
+        and all(s % 8 == 0 for s in x.stride()[:-1])
+    )
+
+
+def _prep_pair(x: torch.Tensor, tx: Optional[torch.Tensor]):
+    """Primal and tangent must end up with identical strides (the kernel reads both through one set)."""
+    if tx is None:
+        return (x if _kernel_ready(x) else x.contiguous()), None
+    if _kernel_ready(x) and _kernel_ready(tx) and x.stride() == tx.stride():
+        return x, tx
+    return x.contiguous(), tx.contiguous()
+
+
+def _strides3(x: torch.Tensor):
+    return (ctypes.c_int64 * 3)(x.stride(0), x.stride(1), x.stride(2))
+
+
+def fwd_jvp(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    tq: Optional[torch.Tensor] = None,
+    tk: Optional[torch.Tensor] = None,
+    tv: Optional[torch.Tensor] = None,
+    causal: bool = False,
+    sm_scale: Optional[float] = None,
+    key_lens: Optional[torch.Tensor] = None,
+    out_layout: str = "bhld",
+    need_lse: bool = True,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """(o, to, lse) for q,k,v (+ tangents) given as ``[B, H, L, d]`` views on one GPU.
+
+    Tangents: none (forward only, ``to`` is None), ``tq`` only, or any mix (missing ones are
+    treated as zeros).  ``out_layout``: "bhld" -> o is contiguous ``[B,H,Lq,dv]``; "blhd" -> the
+    memory is contiguous ``[B,Lq,H,dv]`` and a ``[B,H,Lq,dv]`` view of it is returned.
+    ``key_lens``: optional int32 ``[B]`` device tensor, keys >= key_lens[b] are masked.
+    """
+    assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q, k, v must be [B, H, L, d]"
+    assert q.shape[:-2] == k.shape[:-2] and k.shape[:-2] == v.shape[:-2]
+    assert k.shape[-2] == v.shape[-2] and q.shape[-1] == k.shape[-1]
+    B, H, Lq, d_qk = q.shape
+    Lkv, d_v = v.shape[-2], v.shape[-1]
+    assert d_qk in REFERENCE_HEAD_DIMS and d_v in REFERENCE_HEAD_DIMS
+    if d_qk not in SUPPORTED_HEAD_DIMS or d_v not in SUPPORTED_HEAD_DIMS:
+        raise NotImplementedError(f"head dims ({d_qk}, {d_v}): the HIP kernels are built for {SUPPORTED_HEAD_DIMS}")
+    assert (Lq == Lkv) or (not causal), "Causal cross-attention is currently not supported."
+    if not q.is_cuda:
+        raise RuntimeError("cosmos attention (HIP) needs tensors on a GPU; there is no CPU path")
+    if q.dtype not in _DTYPES:
+        raise NotImplementedError(f"dtype={q.dtype} is not supported (bf16 / fp16)")
+    assert k.dtype == q.dtype and v.dtype == q.dtype
+    assert k.device == q.device and v.device == q.device
+    for t_, x_ in ((tq, q), (tk, k), (tv, v)):
+        if t_ is not None:
+            assert t_.shape == x_.shape and t_.dtype == x_.dtype and t_.device == x_.device
+
+    have_tangent = any(t_ is not None for t_ in (tq, tk, tv))
+    if have_tangent and tq is None:
+        tq = torch.zeros_like(q)
+    if tk is not None or tv is not None:  # kernels are built for: none / q only / all three
+        tk = torch.zeros_like(k) if tk is None else tk
+        tv = torch.zeros_like(v) if tv is None else tv
+    q, tq = _prep_pair(q, tq)
+    k, tk = _prep_pair(k, tk)
+    v, tv = _prep_pair(v, tv)
+
+    if sm_scale is None:
+        sm_scale = d_qk ** (-0.5)
+
+    if out_layout == "bhld":
+        o = torch.empty((B, H, Lq, d_v), device=q.device, dtype=q.dtype)
+    elif out_layout == "blhd":
+        o = torch.empty((B, Lq, H, d_v), device=q.device, dtype=q.dtype).transpose(1, 2)
+    else:
+        raise ValueError(f"out_layout={out_layout!r}")
+    to = torch.empty_like(o) if have_tangent else None  # empty_like keeps o's strides
+    lse = torch.empty((B, H, Lq), device=q.device, dtype=torch.float32) if need_lse else None
+
+    if key_lens is not None:
+        assert not causal, "key_lens with causal is not supported"
+        key_lens = key_lens.to(device=q.device, dtype=torch.int32).contiguous()
+        assert key_lens.shape == (B,)
+
+    desc = _lib.AttnDesc()
+    desc.abi_version = _lib.ABI_VERSION
+    desc.dtype = _DTYPES[q.dtype]
+    desc.B, desc.H, desc.Lq, desc.Lkv, desc.d_qk, desc.d_v = B, H, Lq, Lkv, d_qk, d_v
+    desc.causal = 1 if causal else 0
+    desc.sm_scale = float(sm_scale)
+    desc.q, desc.k, desc.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    desc.tq = tq.data_ptr() if tq is not None else None
+    desc.tk = tk.data_ptr() if tk is not None else None
+    desc.tv = tv.data_ptr() if tv is not None else None
+    desc.q_stride, desc.k_stride, desc.v_stride = _strides3(q), _strides3(k), _strides3(v)
+    desc.o, desc.to = o.data_ptr(), (to.data_ptr() if to is not None else None)
+    desc.o_stride = _strides3(o)
+    desc.lse = lse.data_ptr() if lse is not None else None
+    desc.key_lens = key_lens.data_ptr() if key_lens is not None else None
+
+    lib = _lib.load_library()
+    with torch.cuda.device(q.device):
+        ws_bytes = lib.cosmos_attn_workspace_bytes(ctypes.byref(desc))
+        if ws_bytes == 0:
+            # invalid descriptor: let the launch entry produce the precise status
+            _lib.raise_for_status(lib.cosmos_attn_fwd_jvp(ctypes.byref(desc), None, 0, None) or _lib.ST_BAD_ARG)
+        workspace = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        status = lib.cosmos_attn_fwd_jvp(ctypes.byref(desc), workspace.data_ptr(), ws_bytes, stream)
+    _lib.raise_for_status(status)
+    # workspace / converted inputs are freed to torch's caching allocator here; it is stream-ordered on
+    # the launch stream, so reuse by later work on this stream is safe.
+    return o, to, lse

@@ -1,0 +1,111 @@
+/*
+ * cosmos_attn_hip.h -- C ABI of the MI355X (gfx950) flash-attention forward + forward-mode
+ * JVP (tangent) library.
+ *
+ * Plain C: pointers, sizes, strides, a hipStream_t passed as void*.  No torch types.
+ * Every entry point is asynchronous on the given stream and never synchronises the device.
+ * All device pointers must belong to the current HIP device.
+ *
+ * Reference interfaces replaced (paths relative to the reference checkout):
+ *   JVP = cosmos_predict2/_src/predict2/utils/flash_attention_jvp_triton.py
+ *   ATT = cosmos_predict2/_src/predict2/networks/attention.py
+ */
+#ifndef COSMOS_ATTN_HIP_H
+#define COSMOS_ATTN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define COSMOS_ATTN_ABI_VERSION 1
+#define COSMOS_ATTN_API __attribute__((visibility("default")))
+
+/* element types of q,k,v,tangents and of o,to (lse is always fp32) */
+enum cosmos_attn_dtype {
+    COSMOS_ATTN_BF16 = 0,
+    COSMOS_ATTN_FP16 = 1
+};
+
+/* status codes (0 = ok).  The Python host maps BAD_SHAPE/BAD_STRIDE to AssertionError like the
+ * reference's asserts (JVP:439-448) and UNSUPPORTED to NotImplementedError (ATT:107-108). */
+enum cosmos_attn_status {
+    COSMOS_ATTN_OK = 0,
+    COSMOS_ATTN_BAD_ARG = 1,        /* null pointer / negative size */
+    COSMOS_ATTN_BAD_SHAPE = 2,      /* head dim not in {16,32,64,128}, causal with Lq != Lkv */
+    COSMOS_ATTN_BAD_STRIDE = 3,     /* misaligned base or stride (16-byte rows required) */
+    COSMOS_ATTN_UNSUPPORTED = 4,    /* dtype / head-dim combination not built */
+    COSMOS_ATTN_WORKSPACE_TOO_SMALL = 5,
+    COSMOS_ATTN_LAUNCH_FAILED = 6   /* hipGetLastError() != hipSuccess after a launch */
+};
+
+/*
+ * One attention call.  Tensors are [B, H, L, d] addressed through element strides
+ * (batch, head, row); the innermost (d) stride is 1.  This covers both the heads-first
+ * layout of the JVP entry (JVP:425-431) and a transposed view of the DiT's [B, S, H, D]
+ * tensors (ATT:166-168) without a copy.  Tangents share the strides of their primals
+ * (the reference asserts this, JVP:448).
+ *
+ * Replaces the argument list of the Triton launch JVP:462-496.
+ */
+typedef struct cosmos_attn_desc {
+    int32_t abi_version;     /* COSMOS_ATTN_ABI_VERSION */
+    int32_t dtype;           /* enum cosmos_attn_dtype */
+    int32_t B, H;            /* batch, heads                                   (JVP:489-490) */
+    int32_t Lq, Lkv;         /* query / key sequence lengths                   (JVP:491-492) */
+    int32_t d_qk, d_v;       /* head dims, each in {16,32,64,128}              (JVP:444-445, 256 not built) */
+    int32_t causal;          /* 1: key j visible to query i iff j <= i; needs Lq == Lkv (JVP:446) */
+    float sm_scale;          /* softmax scale; caller resolves the default d_qk^-0.5 (JVP:449-450) */
+
+    const void *q, *k, *v;   /* primals (device) */
+    const void *tq, *tk, *tv;/* tangents (device); all NULL = forward only; tk == tv == NULL = tangent on q only */
+    int64_t q_stride[3];     /* (batch, head, row) element strides of q and tq */
+    int64_t k_stride[3];     /* of k and tk */
+    int64_t v_stride[3];     /* of v and tv */
+
+    void *o, *to;            /* outputs [B,H,Lq,d_v] in `dtype`; `to` may be NULL iff all tangents are NULL */
+    int64_t o_stride[3];     /* (batch, head, row) element strides of o and to (d stride 1) */
+    float *lse;              /* [B,H,Lq] fp32 contiguous: natural-log logsumexp of the scaled scores (JVP:367,376); may be NULL */
+
+    const int32_t *key_lens; /* optional [B] int32 (device): keys >= key_lens[b] are masked out.  No counterpart in the
+                                reference, which never masks (ATT:94-95 ignores k_lens); pinned by the torch oracle. */
+} cosmos_attn_desc;
+
+/* ABI version of the loaded library. */
+COSMOS_ATTN_API int cosmos_attn_abi_version(void);
+
+/* Human-readable text for a status code (static storage). */
+COSMOS_ATTN_API const char *cosmos_attn_status_string(int status);
+
+/*
+ * Bytes of device workspace the call needs (K, V and their tangents re-tiled into the
+ * kernel's LDS image).  0 on invalid descriptors.  The host allocates it however it likes
+ * (the Python host uses torch's caching allocator) and may reuse it across calls on one stream.
+ * No counterpart in the reference (Triton reads K/V in place).
+ */
+COSMOS_ATTN_API size_t cosmos_attn_workspace_bytes(const cosmos_attn_desc *desc);
+
+/*
+ * Forward + JVP:  o = softmax(q k^T s) v ;  to = d/de o(q+e tq, k+e tk, v+e tv)|_{e=0} ;  lse.
+ * Forward only when all tangent pointers are NULL.
+ * Replaces `_attention.forward` -> `_attn_fwd[grid](...)`  (JVP:436-502, JVP:176-378) and, forward only,
+ * the SDPA / FA3 call of `attention()` (ATT:119-127, ATT:170-178).
+ * Launches the re-tiling kernel and the attention kernel on `stream`; returns a status code.
+ */
+COSMOS_ATTN_API int cosmos_attn_fwd_jvp(const cosmos_attn_desc *desc, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * The two stages separately, for callers that reuse K/V across calls (e.g. cross-attention
+ * against a fixed text context, JVP with several tangent directions on q only) and for profiling.
+ *   cosmos_attn_pack_kv : k,v(,tk,tv) -> workspace
+ *   cosmos_attn_run     : q(,tq), workspace -> o(,to), lse     (desc->k/v/tk/tv are only tested for NULL)
+ */
+COSMOS_ATTN_API int cosmos_attn_pack_kv(const cosmos_attn_desc *desc, void *workspace, size_t workspace_bytes, void *stream);
+COSMOS_ATTN_API int cosmos_attn_run(const cosmos_attn_desc *desc, const void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COSMOS_ATTN_HIP_H */
