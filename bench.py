@@ -1,0 +1,212 @@
+"""Benchmark of the attention forward + JVP hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5] [--no-cpu]
+
+A "step" is one call of the hot path (re-tiling kernel + attention kernel, through the Python host and
+the C ABI) over one batch of synthetic tensors that are already resident in HBM.  Default workload: the
+configuration the headline metric is quoted on -- 2B DiT self-attention forward + JVP at the 720p shape,
+B=1, H=16, L=84480, d=128, bf16.  Prints ONE JSON line.
+
+FLOP accounting is the reference's own (cosmos_predict2/_src/predict2/utils/flash_attention_jvp_triton.py:703-713):
+2*B*H*Lq*Lkv*d per matmul, 2 matmuls forward, 6 forward + JVP.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+REPO_ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, REPO_ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+# MI355X dense bf16 MFMA peak: 256 CU x 4096 FLOP/clk/CU x 2.4 GHz
+PEAK_BF16_TFLOPS = 256 * 4096 * 2.4e9 / 1e12
+
+WORKLOADS = {
+    # name: (description, B, H, Lq, Lkv, d, tangents, rms-normed q/k, key-padding)
+    "c2": ("2B DiT self-attention fwd bf16 480p B1 H16 L37440 d128", 1, 16, 37440, 37440, 128, "none", True, False),
+    "c3": ("2B DiT self-attention fwd+JVP bf16 720p B1 H16 L84480 d128", 1, 16, 84480, 84480, 128, "full", False, False),
+    "c4": ("14B DiT self-attention fwd+JVP bf16 720p B1 H40 L84480 d128", 1, 40, 84480, 84480, 128, "full", True, False),
+    "c5": ("2B DiT text cross-attention fwd+JVP bf16 B2 H16 Lq37440 Lkv512 d128 key-padding tangent-on-q", 2, 16, 37440, 512, 128, "q", False, True),
+}
+
+
+def make_device_inputs(B, H, Lq, Lkv, d, tangents, rms, dev, seed=0):
+    """Synthetic tensors generated on the GPU per head block (values ~N(0,1), tangents ~N(0,1)*0.1)."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+
+    def rn(L, std, norm=False):
+        x = torch.randn((B, H, L, d), generator=g, device=dev, dtype=torch.float32) * std
+        if norm:
+            x = x * torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + 1e-6)
+        return x.to(torch.bfloat16)
+
+    q, k, v = rn(Lq, 1.0, rms), rn(Lkv, 1.0, rms), rn(Lkv, 1.0)
+    tq = rn(Lq, 0.1) if tangents != "none" else None
+    tk = rn(Lkv, 0.1) if tangents == "full" else None
+    tv = rn(Lkv, 0.1) if tangents == "full" else None
+    return q, k, v, tq, tk, tv
+
+
+def cpu_baseline(oracle, H, Lkv, d, tangents, rows=512, seed=0):
+    """The reference's CPU path -- torch math SDPA under torch.func.jvp, fp32 -- timed on this host's cores
+    on a bounded sample: `rows` query rows against the full K/V for all heads (query rows are independent,
+    so FLOP/s on the sample is FLOP/s of the whole call)."""
+    q, k, v, tq, tk, tv = oracle.make_inputs((1, H, rows, d), (1, H, Lkv, d), seed=seed, dtype=torch.float32)
+    if tangents == "none":
+        fn = lambda: oracle.sdpa_forward_torch(q, k, v)
+        n_mm = 2
+    else:
+        if tangents == "q":
+            tk = tv = None
+        fn = lambda: oracle.sdpa_jvp_torch(q, k, v, tq, tk, tv)
+        n_mm = 6
+    fn()  # warm-up
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        fn()
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > 10.0 or reps >= 5:
+            break
+    sec = el / reps
+    flops = n_mm * 2.0 * H * rows * Lkv * d
+    return {
+        "value": flops / sec / 1e12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "host_cpus": os.cpu_count(),
+        "kind": "port",
+        "sample": f"torch math SDPA + torch.func.jvp fp32, {rows} query rows x full Lkv={Lkv} x {H} heads, "
+                  f"{reps} reps, {sec:.3f} s per rep; rows are independent so the rate extrapolates to the full call",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calib", action="store_true",
+                    help="also run one plain 1 GiB device copy (calibrates FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the hot path is a single-GPU kernel; "
+              "sharding across GPUs is design-only). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    pkg = entry.load_package()
+    lib = pkg._lib.load_library()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    desc_txt, B, H, Lq, Lkv, d, tangents, rms, padded = WORKLOADS[args.workload]
+    q, k, v, tq, tk, tv = make_device_inputs(B, H, Lq, Lkv, d, tangents, rms, dev)
+    key_lens = None
+    mean_len = Lkv
+    if padded:
+        g = torch.Generator().manual_seed(0)
+        kl = torch.randint(64, Lkv + 1, (B,), generator=g)
+        key_lens = kl.to(device=dev, dtype=torch.int32)
+        mean_len = float(kl.float().mean())
+    n_mm = 2 if tangents == "none" else 6
+    flops = n_mm * 2.0 * B * H * Lq * Lkv * d            # nominal (padded Lkv), the reference's accounting
+    n_mm_alg = {"none": 2, "q": 4, "full": 6}[tangents]  # matmuls that are not identically zero
+    flops_alg = n_mm_alg * 2.0 * B * H * Lq * mean_len * d
+
+    def step():
+        return pkg.fwd_jvp(q, k, v, tq, tk, tv, key_lens=key_lens)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / args.steps
+    del out
+
+    # dominant kernel alone (attn_fwd_jvp_kernel), HIP events on the launch stream, K/V already re-tiled
+    import ctypes
+    from types import SimpleNamespace
+
+    o = torch.empty((B, H, Lq, d), device=dev, dtype=torch.bfloat16)
+    to = torch.empty_like(o) if tangents != "none" else None
+    lse = torch.empty((B, H, Lq), device=dev, dtype=torch.float32)
+    D = pkg._lib.AttnDesc()
+    D.abi_version, D.dtype = pkg._lib.ABI_VERSION, pkg._lib.DTYPE_BF16
+    D.B, D.H, D.Lq, D.Lkv, D.d_qk, D.d_v, D.causal, D.sm_scale = B, H, Lq, Lkv, d, d, 0, d ** -0.5
+    ptr = lambda x: None if x is None else x.data_ptr()
+    D.q, D.k, D.v, D.tq, D.tk, D.tv = ptr(q), ptr(k), ptr(v), ptr(tq), ptr(tk), ptr(tv)
+    s3 = lambda x: (ctypes.c_int64 * 3)(x.stride(0), x.stride(1), x.stride(2))
+    D.q_stride, D.k_stride, D.v_stride, D.o_stride = s3(q), s3(k), s3(v), s3(o)
+    D.o, D.to, D.lse, D.key_lens = ptr(o), ptr(to), ptr(lse), ptr(key_lens)
+    ws_bytes = lib.cosmos_attn_workspace_bytes(ctypes.byref(D))
+    ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
+    stream = torch.cuda.current_stream().cuda_stream
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    pack_ms, run_ms = [], []
+    for i in range(args.warmup + args.steps):
+        e0, e1, e2 = ev(), ev(), ev()
+        e0.record()
+        assert lib.cosmos_attn_pack_kv(ctypes.byref(D), ws.data_ptr(), ws_bytes, stream) == 0
+        e1.record()
+        assert lib.cosmos_attn_run(ctypes.byref(D), ws.data_ptr(), ws_bytes, stream) == 0
+        e2.record()
+        torch.cuda.synchronize()
+        if i >= args.warmup:
+            pack_ms.append(e0.elapsed_time(e1))
+            run_ms.append(e1.elapsed_time(e2))
+    run_avg = sum(run_ms) / len(run_ms)
+    pack_avg = sum(pack_ms) / len(pack_ms)
+    achieved = flops / (run_avg * 1e-3) / 1e12
+
+    result = {
+        "metric": "attn fwd+JVP TFLOP/s & % bf16 MFMA peak @ 2B 720p (L=84480); ms per call",
+        "value": flops / sec / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": sec * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": desc_txt, "B": B, "H": H, "Lq": Lq, "Lkv": Lkv, "d": d,
+                   "tangents": tangents, "flop_per_call": flops,
+                   "pct_of_bf16_mfma_peak": 100.0 * flops / sec / 1e12 / PEAK_BF16_TFLOPS},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "attn_fwd_jvp_kernel", "kernel_ms_avg": run_avg, "kernel_ms_min": min(run_ms),
+                     "pack_kv_kernel_ms_avg": pack_avg},
+    }
+    if padded:
+        result["config"]["mean_key_len"] = mean_len
+        result["config"]["algorithmic_flop_per_call"] = flops_alg
+        result["config"]["algorithmic_tflops"] = flops_alg / sec / 1e12
+    if args.copy_calib:
+        src = torch.empty(1 << 30, device=dev, dtype=torch.uint8).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # one elementwise copy kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+    if not args.no_cpu:
+        del ws, o, to
+        oracle = entry.load_oracle()
+        result["cpu_baseline"] = cpu_baseline(oracle, H, Lkv, d, tangents)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
