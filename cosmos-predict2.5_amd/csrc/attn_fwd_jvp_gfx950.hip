@@ -56,20 +56,32 @@ __device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
 }
 
 constexpr int kBlockM = 128;       // query rows per workgroup (4 wavefronts x 32)
-constexpr int kBlockN = 64;        // keys per tile
+constexpr int kBlockN = 32;        // keys per tile
 constexpr int kThreads = 256;
 constexpr int kFragBytes = 1024;   // one MFMA A-operand fragment: 64 lanes x 16 B
+#ifndef COSMOS_ATTN_PREFETCH_GROUPS
+#define COSMOS_ATTN_PREFETCH_GROUPS 2
+#endif
+#ifndef COSMOS_ATTN_SWEEP_STAGGER
+#define COSMOS_ATTN_SWEEP_STAGGER 2   // tiles between the sweep starts of workgroups that share an L2
+#endif
 
 enum { MODE_FWD = 0, MODE_JVP_Q = 1, MODE_JVP_FULL = 2 };
 
-// Geometry of one packed KV tile ("LDS image").  Sections in order: K, V^T, dK, dV^T (the last two only
-// with tangents on k/v).  K-type fragment (kb, c): lane l holds K[32 kb + l%32][16 c + 8 (l/32) .. +7].
-// V^T-type fragment (db, c): lane l, slot s holds V[16 c + 8 (s/4) + 4 (l/32) + s%4][32 db + l%32].
+// Geometry of one packed KV tile ("LDS image") of kBlockN = 32 keys.  Sections in order: K, dK (the
+// "K part"), V^T, dV^T (the "V part"); dK / dV^T only with tangents on k/v.  Every section is a run of
+// 1 KB MFMA A-operand fragments (64 lanes x 16 B):
+//   K-type fragment c (c < dqk/16):            lane l holds K[l%32][16 c + 8 (l/32) .. +7]
+//   V^T-type fragment (db, c) (c < 2), index 2 db + c:
+//                                              lane l, slot s holds V[16 c + 8 (s/4) + 4 (l/32) + s%4][32 db + l%32]
+// (the key order inside a V^T fragment is the order in which the S^T accumulator registers of
+// v_mfma_f32_32x32x16 hold keys, so P^T needs no shuffle to become the B operand).
 struct TileGeom {
-    int nc, ndb, k_frags, vt_frags, tile_frags;
+    int nc, ndb, k_frags, vt_frags, kpart_frags, tile_frags;
     __host__ __device__ TileGeom(int dqk, int dv, bool full)
-        : nc(dqk / 16), ndb((dv + 31) / 32), k_frags(2 * (dqk / 16)), vt_frags(4 * ((dv + 31) / 32)),
-          tile_frags((2 * (dqk / 16) + 4 * ((dv + 31) / 32)) * (full ? 2 : 1)) {}
+        : nc(dqk / 16), ndb((dv + 31) / 32), k_frags(dqk / 16), vt_frags(2 * ((dv + 31) / 32)),
+          kpart_frags((dqk / 16) * (full ? 2 : 1)),
+          tile_frags(((dqk / 16) + 2 * ((dv + 31) / 32)) * (full ? 2 : 1)) {}
 };
 
 struct PackParams {
@@ -79,38 +91,44 @@ struct PackParams {
     int H, Lkv, dqk, dv, n_tiles;
 };
 
-// grid (n_tiles, B*H); every 16-byte unit of the tile image is produced by one thread.
+// grid (ceil(n_tiles / 2), B*H); every 16-byte unit of a tile image is produced by one thread.
 __global__ void __launch_bounds__(kThreads) pack_kv_kernel(const PackParams p) {
-    const int t = blockIdx.x, bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
+    const int bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
     const bool full = p.tk != nullptr;
     const TileGeom g(p.dqk, p.dv, full);
-    uint4* dst = p.out + ((size_t)bh * p.n_tiles + t) * (size_t)(g.tile_frags * (kFragBytes / 16));
     const int64_t k_off = (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
     const int64_t v_off = (int64_t)b * p.v_sb + (int64_t)h * p.v_sh;
     const int units = g.tile_frags * 64;
-    for (int u = threadIdx.x; u < units; u += kThreads) {
-        int frag = u >> 6;
-        const int l = u & 63, i = l & 31, hh = l >> 5;
-        const uint16_t *ksrc = p.k, *vsrc = p.v;
-        if (frag >= g.k_frags + g.vt_frags) { frag -= g.k_frags + g.vt_frags; ksrc = p.tk; vsrc = p.tv; }
-        uint4 val = make_uint4(0u, 0u, 0u, 0u);
-        if (frag < g.k_frags) {
-            const int kb = frag / g.nc, c = frag % g.nc;
-            const int key = t * kBlockN + 32 * kb + i;
-            if (key < p.Lkv) val = *reinterpret_cast<const uint4*>(ksrc + k_off + (int64_t)key * p.k_sl + 16 * c + 8 * hh);
-        } else {
-            const int f = frag - g.k_frags, db = f >> 2, c = f & 3;
-            const int d = 32 * db + i;
-            uint16_t e[8];
+    for (int tt = 0; tt < 2; ++tt) {
+        const int t = blockIdx.x * 2 + tt;
+        if (t >= p.n_tiles) break;
+        uint4* dst = p.out + ((size_t)bh * p.n_tiles + t) * (size_t)(g.tile_frags * (kFragBytes / 16));
+        for (int u = threadIdx.x; u < units; u += kThreads) {
+            int frag = u >> 6;
+            const int l = u & 63, i = l & 31, hh = l >> 5;
+            uint4 val = make_uint4(0u, 0u, 0u, 0u);
+            if (frag < g.kpart_frags) {
+                const uint16_t* src = p.k;
+                if (frag >= g.k_frags) { frag -= g.k_frags; src = p.tk; }
+                const int key = t * kBlockN + i;
+                if (key < p.Lkv) val = *reinterpret_cast<const uint4*>(src + k_off + (int64_t)key * p.k_sl + 16 * frag + 8 * hh);
+            } else {
+                frag -= g.kpart_frags;
+                const uint16_t* src = p.v;
+                if (frag >= g.vt_frags) { frag -= g.vt_frags; src = p.tv; }
+                const int db = frag >> 1, c = frag & 1;
+                const int d = 32 * db + i;
+                uint16_t e[8];
 #pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                const int key = t * kBlockN + 16 * c + 8 * (s >> 2) + 4 * hh + (s & 3);
-                e[s] = (key < p.Lkv && d < p.dv) ? vsrc[v_off + (int64_t)key * p.v_sl + d] : (uint16_t)0;
+                for (int s = 0; s < 8; ++s) {
+                    const int key = t * kBlockN + 16 * c + 8 * (s >> 2) + 4 * hh + (s & 3);
+                    e[s] = (key < p.Lkv && d < p.dv) ? src[v_off + (int64_t)key * p.v_sl + d] : (uint16_t)0;
+                }
+                val.x = e[0] | ((uint32_t)e[1] << 16); val.y = e[2] | ((uint32_t)e[3] << 16);
+                val.z = e[4] | ((uint32_t)e[5] << 16); val.w = e[6] | ((uint32_t)e[7] << 16);
             }
-            val.x = e[0] | ((uint32_t)e[1] << 16); val.y = e[2] | ((uint32_t)e[3] << 16);
-            val.z = e[4] | ((uint32_t)e[5] << 16); val.w = e[6] | ((uint32_t)e[7] << 16);
+            dst[u] = val;
         }
-        dst[u] = val;
     }
 }
 
@@ -128,26 +146,294 @@ struct AttnParams {
 
 extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-__device__ __forceinline__ void load_tile_to_lds(const char* src_lane, char* dst, int wave, int tile_frags) {
-    // each wavefront-level instruction moves one 1 KB fragment: LDS address = dst + lane * 16
-    for (int f = wave; f < tile_frags; f += 4) {
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src_lane + f * kFragBytes),
-                                         (__attribute__((address_space(3))) void*)(dst + f * kFragBytes), 16, 0, 0);
+#define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// Per-wavefront state and the per-tile work, templated so that everything unrolls into registers.
+template <typename T, int DQK, int DV, int MODE>
+struct AttnWave {
+    typedef typename VecOf<T>::v8 V8;
+    static constexpr int NC = DQK / 16;             // 16-wide d chunks of the QK^T contraction
+    static constexpr int NDB = (DV + 31) / 32;      // 32-row blocks of O^T
+    static constexpr bool JVP = MODE != MODE_FWD, FULL = MODE == MODE_JVP_FULL;
+    static constexpr int K_FR = NC, VT_FR = 2 * NDB;
+    static constexpr int KP_FR = K_FR * (FULL ? 2 : 1), VP_FR = VT_FR * (FULL ? 2 : 1);
+    static constexpr int KP_BYTES = KP_FR * kFragBytes, VP_BYTES = VP_FR * kFragBytes;
+    static constexpr int TILE_BYTES = KP_BYTES + VP_BYTES;
+    static constexpr int DK_OFF = K_FR * kFragBytes;     // inside the K part
+    static constexpr int DVT_OFF = VT_FR * kFragBytes;   // inside the V part
+    static constexpr int KP_LOADS = (KP_FR + 3) / 4, VP_LOADS = (VP_FR + 3) / 4;   // per wavefront per tile
+    static constexpr int GROUP_LOADS = KP_LOADS + VP_LOADS;
+    static constexpr int MFMA_PER_C = FULL ? 3 : (JVP ? 2 : 1);
+    static constexpr int SLOTS = NC * MFMA_PER_C;        // MFMA issue slots of the score stage
+
+    // Scores of one tile as this lane sees them: its query column x 16 of the tile's 32 keys (element e is key
+    // 8 (e/4) + 4 (lane/32) + e%4 of the tile).  Kept as plain floats (VGPRs) between steps; the MFMA
+    // accumulators they are copied from live in AccVGPRs only inside a step.
+    struct Scores { float s[16]; float ds[16]; };
+
+    V8 qf[NC], tqf[NC];                 // (arrays of unused modes are never touched and cost no registers)
+    f32x16 acc[NDB], acct[NDB];
+    static constexpr int PD = COSMOS_ATTN_PREFETCH_GROUPS;   // LDS operand fetches run this many MFMA groups ahead of use
+    V8 pre_a[PD], pre_b[PD];   // LDS fragments of the next step's first PD MFMA groups (fetched ahead)
+    float m_run, l_run, r_run;
+    float scale_log2, sm_scale;
+    int lane;
+
+    // Direct-to-LDS copy of a part (NFR fragments of 1 KB), spread over the 4 wavefronts; every wavefront issues
+    // the same number of loads (surplus ones repeat a fragment) so that vmcnt bookkeeping is uniform.
+    // buffer_load ... lds (MUBUF) rather than global_load_lds: the compiler's wait-count pass treats the latter as
+    // a FLAT access that may touch LDS and then turns every later LDS wait into lgkmcnt(0), which exposes the
+    // full LDS latency of the operand prefetches.  One wavefront-level load moves one fragment: lane l's 16
+    // bytes (voffset = 16 l) land at dst + 16 l.
+    // What one wavefront copies per step (one "load group"): its share of the K part of one tile and of the V part
+    // of another, as KP_LOADS + VP_LOADS wavefront-level loads.
+    struct LoadJob {
+        __amdgpu_buffer_rsrc_t rsrc;
+        int lane_off;            // 16 * lane
+        int k_src, v_src;        // byte offsets of the K part / V part in the packed buffer
+        char *k_dst, *v_dst;     // LDS destinations
+        int wave;
+    };
+    // load number i of the group, 0 <= i < GROUP_LOADS
+    __device__ __forceinline__ static void issue_load(const LoadJob& j, int i) {
+        const bool kpart = i < KP_LOADS;
+        const int n = kpart ? KP_FR : VP_FR;
+        int f = j.wave + 4 * (kpart ? i : i - KP_LOADS);
+        if (n % 4 != 0) f = f % n;   // surplus loads repeat a fragment
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(j.rsrc, (__attribute__((address_space(3))) void*)((kpart ? j.k_dst : j.v_dst) + f * kFragBytes), 16,
+                                                 j.lane_off, (kpart ? j.k_src : j.v_src) + f * kFragBytes, 0, 0);
     }
-}
+    __device__ __forceinline__ static void issue_all(const LoadJob& j) {
+#pragma unroll
+        for (int i = 0; i < GROUP_LOADS; ++i) issue_load(j, i);
+    }
+
+    __device__ __forceinline__ V8 lds_frag(const char* base, int frag) const {
+        return *reinterpret_cast<const V8*>(base + frag * kFragBytes + lane * 16);
+    }
+
+    // Rare path (last tile of a ragged / padded key range, causal diagonal): masked keys (>= kv_len, or above the
+    // diagonal when causal) get score -inf, hence p = 0 and H = 0.  Returns the lane-local max of the masked scores.
+    __device__ __forceinline__ static float mask_scores(Scores& x, int key0, int kv_len, bool causal, int row) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int key = key0 + 8 * (e >> 2) + (e & 3);
+            const bool ok = key < kv_len && (!causal || key <= row);
+            x.s[e] = ok ? x.s[e] : -INFINITY;
+            mx = fmaxf(mx, x.s[e]);
+        }
+        return mx;
+    }
+
+    // scores of one tile with nothing interleaved (prologue); returns the lane-local max of s
+    __device__ __forceinline__ float scores_plain(Scores& x, const char* kpart) const {
+        f32x16 s, ds;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { s[e] = 0.f; ds[e] = 0.f; }
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const V8 kf = lds_frag(kpart, c);
+            if (JVP) ds = mfma32(kf, tqf[c], ds);
+            s = mfma32(kf, qf[c], s);
+            if (FULL) ds = mfma32(lds_frag(kpart + DK_OFF, c), qf[c], ds);
+        }
+        // explicit AccVGPR -> VGPR copies (as in step(), so that the scores carried between steps are VGPR values
+        // for every definition); the wait states after the last MFMA are spelled out
+        // (inside the same asm statements as the reads: a separate nop statement could be scheduled away from them)
+        float mx = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            float sv = s[e];
+            asm volatile("s_nop 15\n\ts_nop 7\n\tv_accvgpr_read_b32 %0, %1" : "=v"(x.s[e]) : "a"(sv));
+            if (JVP) {
+                float dv = ds[e];
+                asm volatile("s_nop 15\n\ts_nop 7\n\tv_accvgpr_read_b32 %0, %1" : "=v"(x.ds[e]) : "a"(dv));
+            }
+            mx = fmaxf(mx, x.s[e]);
+        }
+        return mx;
+    }
+
+    // Softmax of element e of this lane's 16, in two halves so that the VALU work can be spread thinly between
+    // MFMAs:  p = exp2(s c - m), l += p   and   H = p dS s, r += H.   Both are rounded to 16-bit MFMA operands.
+    __device__ __forceinline__ void softmax_p(const Scores& x, float* pv, V8* pf, int e) {
+        pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(x.s[e], scale_log2, -m_run));
+        l_run += pv[e];
+        pf[e >> 3][e & 7] = (T)pv[e];
+    }
+    __device__ __forceinline__ void softmax_h(const Scores& x, const float* pv, V8* hf, int e) {
+        if (JVP) {
+            const float hv = pv[e] * (x.ds[e] * sm_scale);
+            r_run += hv;
+            hf[e >> 3][e & 7] = (T)hv;
+        }
+    }
+
+    // Fold a tile's lane-local score max into the running max; rescale the accumulators when some row's max
+    // moved (wavefront-uniform branch; alpha == 1 exactly otherwise).
+    __device__ __forceinline__ void update_max(float mx) {
+        {   // max with lane ^ 32 (the other half of the same query column): one VALU swap, no LDS round trip
+            const unsigned bits = __builtin_bit_cast(unsigned, mx);
+            const auto sw = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+            mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+        }
+        const float m_new = fmaxf(m_run, mx * scale_log2);
+        if (__any(m_new > m_run)) {
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= alpha;
+            r_run *= alpha;
+            // The accumulators live in AccVGPRs for the whole KV sweep (they are only ever MFMA operands).  This
+            // rare path scales them in place through a scratch VGPR; the "+a" constraints keep the register
+            // allocator from copying all of them to VGPRs around the branch on every step.  The MFMA -> AccVGPR
+            // read and AccVGPR write -> MFMA dependencies are invisible to the compiler inside the asm, so the
+            // required wait states are spelled out as s_nop.
+#pragma unroll
+            for (int i = 0; i < NDB; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    // the first statement of each accumulator carries the MFMA -> read wait states
+                    float x = acc[i][e], tmp;
+                    if (e == 0)
+                        asm volatile("s_nop 15\n\ts_nop 7\n\tv_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 3"
+                                     : "+a"(x), "=&v"(tmp) : "v"(alpha));
+                    else
+                        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 3"
+                                     : "+a"(x), "=&v"(tmp) : "v"(alpha));
+                    acc[i][e] = x;
+                    if (JVP) {
+                        float y = acct[i][e], tmp2;
+                        if (e == 0)
+                            asm volatile("s_nop 15\n\ts_nop 7\n\tv_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 3"
+                                         : "+a"(y), "=&v"(tmp2) : "v"(alpha));
+                        else
+                            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 3"
+                                         : "+a"(y), "=&v"(tmp2) : "v"(alpha));
+                        acct[i][e] = y;
+                    }
+                }
+            }
+            m_run = m_new;
+        }
+    }
+
+    static constexpr int NB = 2 * NDB;      // MFMA groups of stage B, g = c * NDB + db
+    static constexpr int NG = NC + NB;      // MFMA groups of a step: stage A chunk c = i, then stage B group g = i - NC
+
+    // LDS fragments of MFMA group i of a step whose stage A reads `kpart` and whose stage B reads `vpart`
+    __device__ __forceinline__ void fetch_group(int i, const char* kpart, const char* vpart, V8& a, V8& b) const {
+        if (i < NC) {
+            a = lds_frag(kpart, i);
+            if (FULL) b = lds_frag(kpart + DK_OFF, i);
+        } else {
+            const int g = i - NC, c = g / NDB, db = g % NDB;
+            a = lds_frag(vpart, 2 * db + c);
+            if (FULL) b = lds_frag(vpart + DVT_OFF, 2 * db + c);
+        }
+    }
+
+    // One software-pipelined step over tile u (scores in `x`, already folded into m_run):
+    //   stage A: scores of tile u+1 (MFMA) | softmax of the first 8 keys per lane (VALU) | this step's LDS fills;
+    //   stage B, first half:  P.V-type products over those keys (MFMA) | softmax of the other 8 keys (VALU);
+    //   stage B, second half: products over the other keys (MFMA) | copy-out of the new scores to VGPRs.
+    // On return `x` holds the scores of tile u+1; the return value is their lane-local max.
+    // kpart1 / vpart0: K part of tile u+1, V part of tile u (this step); kpart2 / vpart1: those of the next step,
+    // already resident, from which the last PD groups fetch the next step's first fragments -- the stream of LDS
+    // operand fetches (PD groups ahead of use) never drains, not even across the workgroup barrier.
+    // A wavefront hides roughly 5 VALU instructions behind one 8-pass MFMA, so the VALU work is dealt out in
+    // slices of that size; scheduling fences keep the written interleaving.
+    __device__ __forceinline__ float step(Scores& x, const char* kpart1, const char* vpart0, const char* kpart2, const char* vpart1,
+                                          const LoadJob& job) {
+        V8 pf[2], hf[2];
+        float pv[16];
+        V8 fa[NG], fb[NG];
+#pragma unroll
+        for (int i = 0; i < PD; ++i) { fa[i] = pre_a[i]; if (FULL) fb[i] = pre_b[i]; }
+        f32x16 sn, dsn;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { sn[e] = 0.f; dsn[e] = 0.f; }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < NG; ++i) {
+            SCHED_FENCE();
+            // operand fetch for group i + PD (of this step, or of the next one)
+            if (i + PD < NG) fetch_group(i + PD, kpart1, vpart0, fa[i + PD], fb[i + PD]);
+            else fetch_group(i + PD - NG, kpart2, vpart1, pre_a[i + PD - NG], pre_b[i + PD - NG]);
+            if (i < NC) {
+                // ---- stage A, d chunk c = i: S^T, dS^T of tile u+1; softmax of elements [0, 8) ----
+                const int c = i, e0 = c * 8 / NC, e1 = (c + 1) * 8 / NC;
+#pragma unroll
+                for (int k = c * GROUP_LOADS / NC; k < (c + 1) * GROUP_LOADS / NC; ++k) issue_load(job, k);
+                SCHED_FENCE();
+                sn = mfma32(fa[i], qf[c], sn);
+#pragma unroll
+                for (int e = e0; e < e1; ++e) softmax_p(x, pv, pf, e);
+                SCHED_FENCE();
+                if (JVP) {
+                    dsn = mfma32(fa[i], tqf[c], dsn);
+#pragma unroll
+                    for (int e = e0; e < e1; ++e) softmax_h(x, pv, hf, e);
+                    SCHED_FENCE();
+                }
+                if (FULL) dsn = mfma32(fb[i], qf[c], dsn);
+            } else {
+                // ---- stage B, group g: O^T += V^T P^T ; T^T += V^T H^T + dV^T P^T ----
+                const int g = i - NC, c = g / NDB, db = g % NDB;
+                SCHED_FENCE();
+                acc[db] = mfma32(fa[i], pf[c], acc[db]);
+                if (c == 0) {   // first half: softmax of elements [8, 16), p-halves
+#pragma unroll
+                    for (int e = 8 + db * 8 / NDB; e < 8 + (db + 1) * 8 / NDB; ++e) softmax_p(x, pv, pf, e);
+                }
+                SCHED_FENCE();
+                if (JVP) acct[db] = mfma32(fa[i], hf[c], acct[db]);
+                if (c == 0) {   // ... h-halves
+#pragma unroll
+                    for (int e = 8 + db * 8 / NDB; e < 8 + (db + 1) * 8 / NDB; ++e) softmax_h(x, pv, hf, e);
+                }
+                if (JVP) SCHED_FENCE();
+                if (FULL) acct[db] = mfma32(fb[i], pf[c], acct[db]);
+                if (c == 1) {
+                    // Second half: copy-out of the next tile's scores (AccVGPR -> VGPR), a slice per group.  Explicit
+                    // instructions: the copy must happen HERE (in the shadow of the MFMA pipe), not wherever the
+                    // register allocator would otherwise place it.  The hardware does not interlock an AccVGPR read
+                    // against the MFMA that produces the register and the compiler cannot see inside the asm; the
+                    // scores were last written in stage A, NDB full MFMA groups before the first read (plus explicit
+                    // wait states), which exceeds the 8-pass MFMA -> read requirement.
+#pragma unroll
+                    for (int e = db * 16 / NDB; e < (db + 1) * 16 / NDB; ++e) {
+                        float sv = sn[e];
+                        if (e == 0 && NDB * MFMA_PER_C >= 6) asm volatile("s_nop 3\n\tv_accvgpr_read_b32 %0, %1" : "=v"(x.s[e]) : "a"(sv));
+                        else if (e == 0) asm volatile("s_nop 15\n\ts_nop 3\n\tv_accvgpr_read_b32 %0, %1" : "=v"(x.s[e]) : "a"(sv));
+                        else asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x.s[e]) : "a"(sv));
+                        if (JVP) {
+                            float dv = dsn[e];
+                            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x.ds[e]) : "a"(dv));
+                        }
+                        mx = fmaxf(mx, x.s[e]);
+                    }
+                }
+            }
+        }
+        SCHED_FENCE();
+        return mx;
+    }
+};
 
 template <typename T, int DQK, int DV, int MODE>
 __global__ void __attribute__((amdgpu_flat_work_group_size(kThreads, kThreads), amdgpu_waves_per_eu(1, 1)))
 attn_fwd_jvp_kernel(const AttnParams p) {
-    typedef typename VecOf<T>::v8 V8;
+    typedef AttnWave<T, DQK, DV, MODE> W;
+    typedef typename W::V8 V8;
     typedef typename VecOf<T>::v4 V4;
-    constexpr int NC = DQK / 16;             // 16-wide d chunks of the QK^T contraction
-    constexpr int NDB = (DV + 31) / 32;      // 32-row blocks of O^T
-    constexpr bool JVP = MODE != MODE_FWD, FULL = MODE == MODE_JVP_FULL;
-    constexpr int K_FR = 2 * NC, VT_FR = 4 * NDB;
-    constexpr int TILE_FR = (K_FR + VT_FR) * (FULL ? 2 : 1);
-    constexpr int TILE_BYTES = TILE_FR * kFragBytes;
-    constexpr int VT_OFF = K_FR * kFragBytes, DK_OFF = (K_FR + VT_FR) * kFragBytes, DVT_OFF = DK_OFF + K_FR * kFragBytes;
+    constexpr int NC = W::NC, NDB = W::NDB;
+    constexpr bool JVP = W::JVP;
+    constexpr int KP_BYTES = W::KP_BYTES, VP_BYTES = W::VP_BYTES, TILE_BYTES = W::TILE_BYTES;
+    constexpr int NBUF = 4;                              // LDS ring depth for K parts and for V parts
+    constexpr int GROUP_LOADS = W::GROUP_LOADS;   // loads per wavefront in one load group
+    // s_waitcnt immediates: vmcnt(n) with expcnt / lgkmcnt left at their maxima
+    constexpr int WAIT_1_GROUP = (GROUP_LOADS & 15) | ((GROUP_LOADS >> 4) << 14) | 0x0F70;
+    static_assert(3 * GROUP_LOADS + W::KP_LOADS <= 63, "vmcnt range");
 
     const int qt = blockIdx.x, bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
     const int lane = threadIdx.x & 63;
@@ -161,12 +447,52 @@ attn_fwd_jvp_kernel(const AttnParams p) {
     int n_tiles = (kv_len + kBlockN - 1) / kBlockN;
     if (p.causal) { const int lim = (qt * kBlockM + kBlockM + kBlockN - 1) / kBlockN; n_tiles = n_tiles < lim ? n_tiles : lim; }
 
-    const char* kv_lane = p.kv + (size_t)bh * p.n_tiles * TILE_BYTES + lane * 16;
-    if (n_tiles > 0) load_tile_to_lds(kv_lane, smem, wave, TILE_FR);
+    // LDS: ring of NBUF K-part buffers, then ring of NBUF V-part buffers.
+    // Load group G(u) = { K part of the tile at sweep position u+1, V part of the tile at position u }: what step u
+    // needs.  Positions past the end wrap around (that data is loaded but never used) so every wavefront always
+    // issues the same number of loads.
+    char* const kring = smem;
+    char* const vring = smem + NBUF * KP_BYTES;
+    // buffer resource over this (batch, head)'s packed tiles: raw (stride 0), num_records in bytes
+    const __amdgpu_buffer_rsrc_t kv_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(p.kv) + (size_t)bh * p.n_tiles * TILE_BYTES, 0, p.n_tiles * TILE_BYTES, 0x00020000);
+    // Sweep order.  The softmax recurrences do not care in which order the KV tiles arrive, so a workgroup may
+    // start its sweep at any tile and wrap around: position u of the sweep is tile (u + shift) mod n.  Workgroups
+    // that share one XCD's L2 (workgroup ids congruent mod 8) start a few tiles apart, so that the first one to
+    // reach a tile takes the L2 miss and the ones behind it hit.  The shift is a fixed function of the workgroup id:
+    // results are bitwise reproducible from run to run.
+    const int n_sweep = n_tiles > 0 ? n_tiles : 1;
+    const int wg_linear = blockIdx.x + gridDim.x * blockIdx.y;
+    const int shift = (((wg_linear >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
+    auto tile_at = [&](int u) {
+        int t = u + shift;
+        t = t >= n_sweep ? t - n_sweep : t;
+        t = t >= n_sweep ? t - n_sweep : t;
+        return t >= n_sweep ? t % n_sweep : t;   // (only sweeps shorter than the prefetch depth get here)
+    };
+    auto make_job = [&](int u) {
+        const int tk = __builtin_amdgcn_readfirstlane(tile_at(u + 1)), tv = __builtin_amdgcn_readfirstlane(tile_at(u));
+        typename W::LoadJob j;
+        j.rsrc = kv_rsrc; j.lane_off = lane * 16; j.wave = wave;
+        j.k_src = tk * TILE_BYTES; j.k_dst = kring + ((u + 1) % NBUF) * KP_BYTES;
+        j.v_src = tv * TILE_BYTES + KP_BYTES; j.v_dst = vring + (u % NBUF) * VP_BYTES;
+        return j;
+    };
+    {   // K part of the first tile of the sweep (as the K half of a pseudo group "-1"), then groups 0..2
+        typename W::LoadJob j = make_job(0);
+        j.k_src = tile_at(0) * TILE_BYTES; j.k_dst = kring;
+#pragma unroll
+        for (int i = 0; i < W::KP_LOADS; ++i) W::issue_load(j, i);
+    }
+    W::issue_all(make_job(0));
+    W::issue_all(make_job(1));
+    W::issue_all(make_job(2));
 
-    // Q (and dQ) fragments: B operand of S^T = K Q^T; lane holds Q[row][16 c + 8 hh .. +7]
-    V8 qf[NC], tqf[JVP ? NC : 1];
-    {
+    W w;
+    w.lane = lane;
+    w.scale_log2 = p.scale_log2;
+    w.sm_scale = p.sm_scale;
+    {   // Q (and dQ) fragments: B operand of S^T = K Q^T; lane holds Q[row][16 c + 8 hh .. +7]
         const int64_t off = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh + (int64_t)row * p.q_sl + 8 * hh;
         const T* qp = reinterpret_cast<const T*>(p.q) + off;
         const T* tqp = reinterpret_cast<const T*>(p.tq) + off;
@@ -174,117 +500,56 @@ attn_fwd_jvp_kernel(const AttnParams p) {
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             V8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-            qf[c] = live ? *reinterpret_cast<const V8*>(qp + 16 * c) : z;
-            if (JVP) tqf[c] = live ? *reinterpret_cast<const V8*>(tqp + 16 * c) : z;
+            w.qf[c] = live ? *reinterpret_cast<const V8*>(qp + 16 * c) : z;
+            if (JVP) w.tqf[c] = live ? *reinterpret_cast<const V8*>(tqp + 16 * c) : z;
         }
     }
-
-    f32x16 acc[NDB], acct[JVP ? NDB : 1];
 #pragma unroll
     for (int i = 0; i < NDB; ++i) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) { acc[i][e] = 0.f; if (JVP) acct[i][e] = 0.f; }
+        for (int e = 0; e < 16; ++e) { w.acc[i][e] = 0.f; if (JVP) w.acct[i][e] = 0.f; }
     }
-    float m_run = -INFINITY;   // running row max of the scaled scores in the log2 domain (same in lanes l, l^32)
-    float l_run = 0.f;         // this lane's partial row sum of p   (the two half-rows are added in the epilogue)
-    float r_run = 0.f;         // this lane's partial row sum of H
+    w.m_run = -INFINITY;   // running row max of the scaled scores, log2 domain (same in lanes l and l^32)
+    w.l_run = 0.f;         // this lane's partial row sum of p (the two half rows are added in the epilogue)
+    w.r_run = 0.f;         // this lane's partial row sum of H
 
-    for (int t = 0; t < n_tiles; ++t) {
-        const char* buf = smem + (t & 1) * TILE_BYTES;
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's share of tile t has landed
-        __syncthreads();                      // everyone's share landed; everyone is done with the other buffer
-        if (t + 1 < n_tiles) load_tile_to_lds(kv_lane + (size_t)(t + 1) * TILE_BYTES, smem + ((t + 1) & 1) * TILE_BYTES, wave, TILE_FR);
+    const bool causal = p.causal != 0;
+    // wavefront-uniform: does tile u hold a key some row of this wavefront must not see?
+    auto need_mask = [&](int t) { return (t * kBlockN + kBlockN > kv_len) || (causal && (t * kBlockN + kBlockN - 1 > row0)); };
 
-        // ---- stage 1: S^T = K Q^T, dS^T = K dQ^T + dK Q^T for 2 blocks of 32 keys ----
-        f32x16 s[2], ds[JVP ? 2 : 1];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) { s[kb][e] = 0.f; if (JVP) ds[kb][e] = 0.f; }
-        }
-#pragma unroll
-        for (int c = 0; c < NC; ++c) {
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                const V8 kf = *reinterpret_cast<const V8*>(buf + (kb * NC + c) * kFragBytes + lane * 16);
-                s[kb] = mfma32(kf, qf[c], s[kb]);
-                if (JVP) ds[kb] = mfma32(kf, tqf[c], ds[kb]);
-                if (FULL) {
-                    const V8 dkf = *reinterpret_cast<const V8*>(buf + DK_OFF + (kb * NC + c) * kFragBytes + lane * 16);
-                    ds[kb] = mfma32(dkf, qf[c], ds[kb]);
-                }
-            }
-        }
+    typename W::Scores sc;
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): everything issued so far has landed (this wavefront's share)
+    __syncthreads();
+    {
+        float mx = w.scores_plain(sc, kring);
+        const int t0 = tile_at(0);
+        if (need_mask(t0)) mx = W::mask_scores(sc, t0 * kBlockN + 4 * hh, kv_len, causal, row);
+        if (n_tiles > 0) w.update_max(mx);
+    }
 
-        // ---- stage 2: online softmax on this lane's query column (32 of the tile's 64 keys) ----
-        // register e of block kb is key  t*64 + 32 kb + 8 (e/4) + 4 hh + e%4
-        const int key0 = t * kBlockN + 4 * hh;
-        const bool need_mask = (t * kBlockN + kBlockN > kv_len) || (p.causal && (t * kBlockN + kBlockN - 1 > row0));
-        if (need_mask) {
+    // fragments of step 0's first two MFMA groups
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int key = key0 + 32 * kb + 8 * (e >> 2) + (e & 3);
-                    const bool ok = key < kv_len && (!p.causal || key <= row);
-                    s[kb][e] = ok ? s[kb][e] : -INFINITY;
-                }
-            }
-        }
-        float mx = s[0][0];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[kb][e]);
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx * p.scale_log2);
-        if (__any(m_new > m_run)) {   // wavefront-uniform: skip the rescale when no row's max moved (alpha == 1 exactly)
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-            l_run *= alpha;
-            r_run *= alpha;
-#pragma unroll
-            for (int i = 0; i < NDB; ++i) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) { acc[i][e] *= alpha; if (JVP) acct[i][e] *= alpha; }
-            }
-            m_run = m_new;
-        }
-        V8 pf[4], hf[JVP ? 4 : 1];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][e], p.scale_log2, -m_run));
-                l_run += pv;
-                pf[2 * kb + (e >> 3)][e & 7] = (T)pv;
-                if (JVP) {
-                    const float hv = pv * (ds[kb][e] * p.sm_scale);
-                    r_run += hv;
-                    hf[2 * kb + (e >> 3)][e & 7] = (T)hv;
-                }
-            }
-        }
+    for (int i = 0; i < W::PD; ++i) w.fetch_group(i, kring + KP_BYTES, vring, w.pre_a[i], w.pre_b[i]);
 
-        // ---- stage 3: O^T += V^T P^T ;  T^T += V^T H^T + dV^T P^T ----
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-#pragma unroll
-            for (int db = 0; db < NDB; ++db) {
-                const V8 vf = *reinterpret_cast<const V8*>(buf + VT_OFF + (db * 4 + c) * kFragBytes + lane * 16);
-                acc[db] = mfma32(vf, pf[c], acc[db]);
-                if (JVP) acct[db] = mfma32(vf, hf[c], acct[db]);
-                if (FULL) {
-                    const V8 dvf = *reinterpret_cast<const V8*>(buf + DVT_OFF + (db * 4 + c) * kFragBytes + lane * 16);
-                    acct[db] = mfma32(dvf, pf[c], acct[db]);
-                }
-            }
+    // Step u: K parts of tiles u+1, u+2 and V parts of tiles u, u+1 are resident (groups u, u+1); group u+2 is in
+    // flight; group u+3 is issued during the step.
+    for (int u = 0; u < n_tiles; ++u) {
+        __builtin_amdgcn_s_waitcnt(WAIT_1_GROUP);    // group u+1 landed (this wavefront's share)
+        __syncthreads();                             // ... everyone's share did, and everyone finished step u-1
+        // group u+3 overwrites the K part of tile u and the V part of tile u-1, both dead since the barrier
+        float mx = w.step(sc, kring + ((u + 1) % NBUF) * KP_BYTES, vring + (u % NBUF) * VP_BYTES,
+                          kring + ((u + 2) % NBUF) * KP_BYTES, vring + ((u + 1) % NBUF) * VP_BYTES, make_job(u + 3));
+        if (u + 1 < n_tiles) {
+            const int tn = tile_at(u + 1);
+            if (need_mask(tn)) mx = W::mask_scores(sc, tn * kBlockN + 4 * hh, kv_len, causal, row);
+            w.update_max(mx);
         }
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // drain the (unused) trailing loads before the LDS is released
 
     // ---- epilogue: O = acc / l ; dO = (T - r O) / l ; LSE = (m + log2 l) ln 2 ----
-    const float l_tot = l_run + __shfl_xor(l_run, 32);
-    const float r_tot = r_run + __shfl_xor(r_run, 32);
+    const float l_tot = w.l_run + __shfl_xor(w.l_run, 32);
+    const float r_tot = w.r_run + __shfl_xor(w.r_run, 32);
     const float inv_l = 1.0f / l_tot;
     const float r_over_l = r_tot * inv_l;
     if (row < p.Lq) {
@@ -300,16 +565,16 @@ attn_fwd_jvp_kernel(const AttnParams p) {
                     V4 ov, tov;
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        const float of = acc[db][4 * g + r] * inv_l;
+                        const float of = w.acc[db][4 * g + r] * inv_l;
                         ov[r] = (T)of;
-                        if (JVP) tov[r] = (T)((acct[db][4 * g + r] - r_over_l * acc[db][4 * g + r]) * inv_l);
+                        if (JVP) tov[r] = (T)((w.acct[db][4 * g + r] - r_over_l * w.acc[db][4 * g + r]) * inv_l);
                     }
                     *reinterpret_cast<V4*>(op + d) = ov;
                     if (JVP) *reinterpret_cast<V4*>(top + d) = tov;
                 }
             }
         }
-        if (p.lse && hh == 0) p.lse[(int64_t)bh * p.Lq + row] = (m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
+        if (p.lse && hh == 0) p.lse[(int64_t)bh * p.Lq + row] = (w.m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
     }
 }
 
@@ -336,6 +601,9 @@ attn_kernel_t pick_dv(int dv, int mode) {
 }
 template <typename T>
 attn_kernel_t pick_dqk(int dqk, int dv, int mode) {
+#ifdef COSMOS_ATTN_ONLY_D128   // development builds: instantiate the d=128 kernels only
+    return (dqk == 128 && dv == 128) ? pick_mode<T, 128, 128>(mode) : nullptr;
+#endif
     switch (dqk) {
         case 16: return pick_dv<T, 16>(dv, mode);
         case 32: return pick_dv<T, 32>(dv, mode);
@@ -355,6 +623,14 @@ int mode_of(const cosmos_attn_desc* d) {
     if (d->tq && d->tk && d->tv) return MODE_JVP_FULL;
     return -1;
 }
+
+size_t tile_bytes_of(const cosmos_attn_desc* d) {
+    const TileGeom g(d->d_qk, d->d_v, mode_of(d) == MODE_JVP_FULL);
+    return (size_t)g.tile_frags * kFragBytes;
+}
+int n_tiles_of(const cosmos_attn_desc* d) { return (d->Lkv + kBlockN - 1) / kBlockN; }
+// workspace = packed tiles [B*H][n_tiles][tile bytes]
+size_t tiles_bytes_of(const cosmos_attn_desc* d) { return (size_t)d->B * d->H * n_tiles_of(d) * tile_bytes_of(d); }
 
 int validate(const cosmos_attn_desc* d) {
     if (!d) return COSMOS_ATTN_BAD_ARG;
@@ -376,14 +652,10 @@ int validate(const cosmos_attn_desc* d) {
     if (!strides_ok(d->q_stride) || !strides_ok(d->k_stride) || !strides_ok(d->v_stride) || !strides_ok(d->o_stride))
         return COSMOS_ATTN_BAD_STRIDE;
     if ((int64_t)d->B * d->H > 65535) return COSMOS_ATTN_BAD_SHAPE;   // grid.y limit
+    if ((int64_t)n_tiles_of(d) * (int64_t)tile_bytes_of(d) >= (int64_t)1 << 31) return COSMOS_ATTN_BAD_SHAPE;   // 32-bit buffer offsets per head
     return COSMOS_ATTN_OK;
 }
 
-size_t tile_bytes_of(const cosmos_attn_desc* d) {
-    const TileGeom g(d->d_qk, d->d_v, mode_of(d) == MODE_JVP_FULL);
-    return (size_t)g.tile_frags * kFragBytes;
-}
-int n_tiles_of(const cosmos_attn_desc* d) { return (d->Lkv + kBlockN - 1) / kBlockN; }
 
 }  // namespace
 
@@ -406,7 +678,7 @@ COSMOS_ATTN_API const char* cosmos_attn_status_string(int status) {
 
 COSMOS_ATTN_API size_t cosmos_attn_workspace_bytes(const cosmos_attn_desc* d) {
     if (validate(d) != COSMOS_ATTN_OK) return 0;
-    return (size_t)d->B * d->H * n_tiles_of(d) * tile_bytes_of(d);
+    return tiles_bytes_of(d);
 }
 
 COSMOS_ATTN_API int cosmos_attn_pack_kv(const cosmos_attn_desc* d, void* workspace, size_t workspace_bytes, void* stream) {
@@ -421,7 +693,7 @@ COSMOS_ATTN_API int cosmos_attn_pack_kv(const cosmos_attn_desc* d, void* workspa
     pp.v_sb = d->v_stride[0]; pp.v_sh = d->v_stride[1]; pp.v_sl = d->v_stride[2];
     pp.out = (uint4*)workspace;
     pp.H = d->H; pp.Lkv = d->Lkv; pp.dqk = d->d_qk; pp.dv = d->d_v; pp.n_tiles = n_tiles_of(d);
-    hipLaunchKernelGGL(pack_kv_kernel, dim3(pp.n_tiles, d->B * d->H), dim3(kThreads), 0, (hipStream_t)stream, pp);
+    hipLaunchKernelGGL(pack_kv_kernel, dim3((pp.n_tiles + 1) / 2, d->B * d->H), dim3(kThreads), 0, (hipStream_t)stream, pp);
     return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
 }
 
@@ -443,7 +715,7 @@ COSMOS_ATTN_API int cosmos_attn_run(const cosmos_attn_desc* d, const void* works
     ap.key_lens = d->key_lens;
     ap.H = d->H; ap.Lq = d->Lq; ap.Lkv = d->Lkv; ap.n_tiles = n_tiles_of(d); ap.causal = d->causal;
     ap.sm_scale = d->sm_scale; ap.scale_log2 = d->sm_scale * 1.4426950408889634f;
-    const size_t lds = 2 * tile_bytes_of(d);
+    const size_t lds = 4 * tile_bytes_of(d);   // rings of 4 K parts + 4 V parts
     if (hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
         (void)hipGetLastError();
         return COSMOS_ATTN_LAUNCH_FAILED;
