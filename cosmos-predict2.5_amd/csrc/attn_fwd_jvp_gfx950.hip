@@ -463,7 +463,9 @@ attn_fwd_jvp_kernel(const AttnParams p) {
     // results are bitwise reproducible from run to run.
     const int n_sweep = n_tiles > 0 ? n_tiles : 1;
     const int wg_linear = blockIdx.x + gridDim.x * blockIdx.y;
-    const int shift = (((wg_linear >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
+    // (not with causal masking: there the first tile of the sweep must be tile 0, the one tile in which every query row
+    // sees a key, so that the running max is finite from the first step on)
+    const int shift = p.causal ? 0 : (((wg_linear >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
     auto tile_at = [&](int u) {
         int t = u + shift;
         t = t >= n_sweep ? t - n_sweep : t;

@@ -1,0 +1,135 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports what the header declares, descriptor
+validation returns the documented status codes (validation happens before anything touches the device), and the
+Python operators raise the same exception types as the reference for the same misuse."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import __graft_entry__ as entry
+
+HEADER = os.path.join(entry.REPO_ROOT, "include", "cosmos_attn_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    return re.findall(r"COSMOS_ATTN_API\s+[\w\s\*]+?\b(cosmos_attn_\w+)\s*\(", text)
+
+
+def test_header_and_binding_agree(pkg):
+    syms = declared_symbols()
+    assert len(syms) >= 6
+    assert sorted(syms) == sorted(pkg._lib.EXPORTS)
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    lib = ctypes.CDLL(pkg._lib.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+    assert pkg._lib.load_library().cosmos_attn_abi_version() == pkg._lib.ABI_VERSION
+    m = re.search(r"#define COSMOS_ATTN_ABI_VERSION (\d+)", open(HEADER).read())
+    assert int(m.group(1)) == pkg._lib.ABI_VERSION
+
+
+def test_desc_struct_layout_matches_header(pkg):
+    # 10 x int32/float, 6 pointers, 9 int64, 2 pointers, 3 int64, 2 pointers
+    assert ctypes.sizeof(pkg._lib.AttnDesc) == 40 + 6 * 8 + 9 * 8 + 2 * 8 + 3 * 8 + 2 * 8
+    assert pkg._lib.AttnDesc.q.offset == 40 and pkg._lib.AttnDesc.key_lens.offset == 208
+
+
+def good_desc(pkg, **over):
+    D = pkg._lib.AttnDesc()
+    D.abi_version, D.dtype = pkg._lib.ABI_VERSION, pkg._lib.DTYPE_BF16
+    D.B, D.H, D.Lq, D.Lkv, D.d_qk, D.d_v, D.causal, D.sm_scale = 1, 2, 100, 70, 128, 64, 0, 0.1
+    fake = 0x7F0000000000  # never dereferenced: validation only looks at values
+    D.q, D.k, D.v, D.o = fake, fake + 4096, fake + 8192, fake + 12288
+    D.tq = D.tk = D.tv = D.to = None
+    for name, sl in (("q_stride", (2 * 100 * 128, 100 * 128, 128)), ("k_stride", (2 * 70 * 128, 70 * 128, 128)),
+                     ("v_stride", (2 * 70 * 64, 70 * 64, 64)), ("o_stride", (2 * 100 * 64, 100 * 64, 64))):
+        setattr(D, name, (ctypes.c_int64 * 3)(*sl))
+    for key, val in over.items():
+        setattr(D, key, val)
+    return D
+
+
+def test_status_codes_for_bad_descriptors(pkg):
+    L, lib = pkg._lib, pkg._lib.load_library()
+    ws = lambda D: lib.cosmos_attn_workspace_bytes(ctypes.byref(D))
+    run = lambda D: lib.cosmos_attn_fwd_jvp(ctypes.byref(D), None, 0, None)
+    D = good_desc(pkg)
+    # forward only: tiles of 32 keys, K part 8 KB + V part (64 -> 2 row blocks) 4 KB
+    assert ws(D) == 1 * 2 * 3 * (8 + 4) * 1024
+    assert run(D) == L.ST_WORKSPACE          # valid descriptor, no workspace: refused before any launch
+    fake = 0x7F0000100000
+    assert ws(good_desc(pkg, tq=fake, tk=fake, tv=fake, to=fake)) == 1 * 2 * 3 * 2 * (8 + 4) * 1024
+    cases = [
+        (dict(abi_version=99), L.ST_BAD_ARG),
+        (dict(Lq=0), L.ST_BAD_ARG),
+        (dict(q=None), L.ST_BAD_ARG),
+        (dict(tk=fake), L.ST_BAD_ARG),                 # tangent on k without q, v
+        (dict(tq=fake), L.ST_BAD_ARG),                 # tangents given but no `to`
+        (dict(dtype=7), L.ST_UNSUPPORTED),
+        (dict(d_qk=256), L.ST_UNSUPPORTED),
+        (dict(d_v=48), L.ST_BAD_SHAPE),
+        (dict(causal=1), L.ST_BAD_SHAPE),              # causal needs Lq == Lkv
+        (dict(q=0x7F0000000008), L.ST_BAD_STRIDE),     # 8-byte aligned base
+        (dict(k_stride=(ctypes.c_int64 * 3)(70 * 132, 70 * 132, 132)), L.ST_BAD_STRIDE),
+    ]
+    for over, want in cases:
+        D = good_desc(pkg, **over)
+        assert ws(D) == 0, over
+        assert run(D) == want, (over, run(D))
+        assert lib.cosmos_attn_pack_kv(ctypes.byref(D), None, 0, None) == want
+        assert lib.cosmos_attn_run(ctypes.byref(D), None, 0, None) == want
+    for st in range(7):
+        assert len(L.status_string(st)) > 0
+    assert L.status_string(0) == "ok"
+
+
+def test_status_to_exception_mapping(pkg):
+    L = pkg._lib
+    L.raise_for_status(L.ST_OK)
+    for st, exc in ((L.ST_BAD_SHAPE, AssertionError), (L.ST_BAD_STRIDE, AssertionError), (L.ST_UNSUPPORTED, NotImplementedError),
+                    (L.ST_BAD_ARG, ValueError), (L.ST_WORKSPACE, RuntimeError), (L.ST_LAUNCH, RuntimeError)):
+        with pytest.raises(exc):
+            L.raise_for_status(st)
+
+
+def test_python_argument_checks_mirror_reference(pkg):
+    q = torch.zeros(1, 2, 8, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):          # no CPU path, no fallback
+        pkg.fwd_jvp(q, q, q)
+    with pytest.raises(AssertionError):                     # shape checks of _attention.forward (…jvp_triton.py:439-440)
+        pkg.fwd_jvp(q, q[:, :1], q)
+    with pytest.raises(AssertionError):
+        pkg.fwd_jvp(q, q, q[:, :, :4])
+    with pytest.raises(AssertionError):                     # head dim outside {16,32,64,128,256} (:444-445)
+        pkg.fwd_jvp(q[..., :48], q[..., :48], q)
+    with pytest.raises(NotImplementedError):                # 256 is accepted by the reference but not built here
+        pkg.fwd_jvp(torch.zeros(1, 1, 8, 256, dtype=torch.bfloat16), torch.zeros(1, 1, 8, 256, dtype=torch.bfloat16), q[:, :1])
+    with pytest.raises(AssertionError, match="Causal cross-attention"):   # :446
+        pkg.fwd_jvp(q, q[:, :, :4], q[:, :, :4], causal=True)
+    with pytest.raises(AssertionError):                     # tangent shape / stride must match the primal (:447-448)
+        pkg.attention_jvp(q, q, q, q[:, :, :4], q, q)
+    with pytest.raises(AssertionError):
+        pkg.attention_jvp(q, q, q, q.transpose(1, 2).contiguous().transpose(1, 2), q, q)
+    with pytest.raises(NotImplementedError):                # attention(): dtype not in the supported list (attention.py:107-108)
+        pkg.attention_forward(q.transpose(1, 2), q.transpose(1, 2), q.transpose(1, 2), dtype=torch.float64)
+    with pytest.raises(NotImplementedError):
+        pkg.attention_forward(q.transpose(1, 2), q.transpose(1, 2), q.transpose(1, 2), dropout_p=0.1)
+
+
+def test_attn_op_refuses_multi_gpu_group(pkg):
+    op = pkg.HipAttnOp()
+    op.set_context_parallel_group(None, None, None)   # single GPU: accepted, as a2a_cp.py:189-193
+    assert op.pg is None
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(entry.REPO_ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr
