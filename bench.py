@@ -28,6 +28,11 @@ import __graft_entry__ as entry  # noqa: E402
 # MI355X dense bf16 MFMA peak: 256 CU x 4096 FLOP/clk/CU x 2.4 GHz
 PEAK_BF16_TFLOPS = 256 * 4096 * 2.4e9 / 1e12
 
+# HBM-side bytes per launch of attn_fwd_jvp_kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# file (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB; factors calibrated with the 1 GiB copy of --copy-calib).
+# Summaries: profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt.  None = not profiled.
+MEASURED_TRAFFIC_BYTES = {"c3": (2 * 2.35761e8 + 681120) * 1024}
+
 WORKLOADS = {
     # name: (description, B, H, Lq, Lkv, d, tangents, rms-normed q/k, key-padding)
     "c2": ("2B DiT self-attention fwd bf16 480p B1 H16 L37440 d128", 1, 16, 37440, 37440, 128, "none", True, False),
@@ -187,7 +192,7 @@ def main():
                    "tangents": tangents, "flop_per_call": flops,
                    "pct_of_bf16_mfma_peak": 100.0 * flops / sec / 1e12 / PEAK_BF16_TFLOPS},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel": "attn_fwd_jvp_kernel", "kernel_ms_avg": run_avg, "kernel_ms_min": min(run_ms),
                      "pack_kv_kernel_ms_avg": pack_avg},
     }

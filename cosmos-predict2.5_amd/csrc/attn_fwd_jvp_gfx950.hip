@@ -18,18 +18,25 @@
 //     fp32 S^T registers, once converted to 16-bit, ARE the B operand of O^T = V^T P^T -- no LDS or
 //     cross-lane shuffle between the two GEMM stages.
 //   * K, V (and dK, dV) are re-tiled ONCE per call by `pack_kv_kernel` into "LDS images": for every
-//     64-key tile, the exact byte order in which the MFMA A-operand fragments are consumed
+//     32-key tile, the exact byte order in which the MFMA A-operand fragments are consumed
 //     (1 KB per fragment = 64 lanes x 16 B, V already transposed and key-permuted to match the
-//     S^T register layout).  The attention kernel then moves tiles HBM/L2 -> LDS with direct-to-LDS
-//     loads (global_load_lds_dwordx4, no VGPR staging) and reads fragments back with conflict-free
-//     linear ds_read_b128.  Re-tiling costs one extra read+write of K/V (<1 % of the call at L=84480)
-//     and removes every transpose / swizzle / tail check from the hot loop.
+//     S^T register layout).  The attention kernel then moves tiles L2 -> LDS with direct-to-LDS
+//     buffer loads (buffer_load_dwordx4 ... lds, no VGPR staging) and reads fragments back with
+//     conflict-free linear ds_read_b128.  Re-tiling costs one extra read+write of K/V (<1 % of the
+//     call at L=84480) and removes every transpose / swizzle / tail check from the hot loop.
 //   * One workgroup = 4 wavefronts = 128 query rows; 1 wavefront per SIMD with the full 512-register
-//     budget (Q, dQ fragments and both fp32 accumulators stay in registers for the whole KV sweep);
-//     LDS holds two tile buffers (2 x 64 KB at d=128 with tangents) so the next tile streams in while
-//     the current one is consumed; one workgroup barrier per tile.
+//     budget: Q, dQ fragments in VGPRs, both fp32 accumulators pinned to AccVGPRs for the whole sweep.
+//   * The KV sweep is software-pipelined in 32-key steps.  Stage A of a step issues the score MFMAs of
+//     the NEXT tile interleaved with the softmax VALU work of the current one; stage B issues the
+//     P.V-type MFMAs of the current tile interleaved with the rest of the softmax and the AccVGPR ->
+//     VGPR copy-out of the next tile's scores.  LDS holds a ring of four K parts and four V parts
+//     (128 KB at d=128 with tangents); every wavefront issues its quarter of the fills three tiles
+//     ahead, waits with s_waitcnt vmcnt(n) for its own fills of the tile needed next, and one workgroup
+//     barrier per step publishes them.  MFMA operands are prefetched from LDS two MFMA groups ahead,
+//     across step boundaries.
 //   * Query-tile index is the fastest grid dimension, so the 256 workgroups in flight sweep the same
-//     head's K/V images together and share them through the per-XCD L2s and the Infinity Cache.
+//     head's K/V images and share them through the per-XCD L2s and the Infinity Cache; workgroups of
+//     one XCD start their (order-free) sweep a few tiles apart so they do not hit one L2 channel at once.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stddef.h>
