@@ -11,7 +11,10 @@ import os
 
 import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 
-from .build import LIB_PATH
+from .build import LIB_PATH as _BUILT_LIB_PATH
+
+# COSMOS_ATTN_LIB: load another build of the same ABI instead of the in-tree one (deployments, A/B timing)
+LIB_PATH = os.environ.get("COSMOS_ATTN_LIB") or _BUILT_LIB_PATH
 
 ABI_VERSION = 1
 DTYPE_BF16, DTYPE_FP16 = 0, 1

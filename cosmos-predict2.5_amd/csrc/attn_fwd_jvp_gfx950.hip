@@ -193,22 +193,34 @@ struct AttnWave {
     // full LDS latency of the operand prefetches.  One wavefront-level load moves one fragment: lane l's 16
     // bytes (voffset = 16 l) land at dst + 16 l.
     // What one wavefront copies per step (one "load group"): its share of the K part of one tile and of the V part
-    // of another, as KP_LOADS + VP_LOADS wavefront-level loads.
+    // of another, as KP_LOADS + VP_LOADS wavefront-level loads.  The share is a contiguous run of fragments
+    // (fragments wave * LOADS .. + LOADS - 1; parts of fewer than 4 fragments are copied redundantly), so one LDS
+    // base (M0) and one scalar offset serve the whole run and the fragment index travels in the instruction's
+    // immediate offset, which is added to both the memory address and the LDS address.
     struct LoadJob {
         __amdgpu_buffer_rsrc_t rsrc;
         int lane_off;            // 16 * lane
-        int k_src, v_src;        // byte offsets of the K part / V part in the packed buffer
-        char *k_dst, *v_dst;     // LDS destinations
-        int wave;
+        int k_src, v_src;        // byte offsets of this wavefront's runs in the packed buffer
+        char *k_dst, *v_dst;     // LDS destinations of the runs
     };
-    // load number i of the group, 0 <= i < GROUP_LOADS
+    __device__ __forceinline__ static int k_run(int wave) { return ((wave * KP_LOADS) % KP_FR) * kFragBytes; }
+    __device__ __forceinline__ static int v_run(int wave) { return ((wave * VP_LOADS) % VP_FR) * kFragBytes; }
+    template <int IMM>
+    __device__ __forceinline__ static void lds_load(__amdgpu_buffer_rsrc_t rsrc, char* dst, int lane_off, int src) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane_off, src, IMM, 0);
+    }
+    // load number i of the group, 0 <= i < GROUP_LOADS (i is a compile-time constant after unrolling; at most 4
+    // loads per part: a part has at most 16 fragments)
     __device__ __forceinline__ static void issue_load(const LoadJob& j, int i) {
         const bool kpart = i < KP_LOADS;
-        const int n = kpart ? KP_FR : VP_FR;
-        int f = j.wave + 4 * (kpart ? i : i - KP_LOADS);
-        if (n % 4 != 0) f = f % n;   // surplus loads repeat a fragment
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(j.rsrc, (__attribute__((address_space(3))) void*)((kpart ? j.k_dst : j.v_dst) + f * kFragBytes), 16,
-                                                 j.lane_off, (kpart ? j.k_src : j.v_src) + f * kFragBytes, 0, 0);
+        char* dst = kpart ? j.k_dst : j.v_dst;
+        const int src = kpart ? j.k_src : j.v_src;
+        switch (kpart ? i : i - KP_LOADS) {
+            case 0: lds_load<0>(j.rsrc, dst, j.lane_off, src); break;
+            case 1: lds_load<1 * kFragBytes>(j.rsrc, dst, j.lane_off, src); break;
+            case 2: lds_load<2 * kFragBytes>(j.rsrc, dst, j.lane_off, src); break;
+            default: lds_load<3 * kFragBytes>(j.rsrc, dst, j.lane_off, src); break;
+        }
     }
     __device__ __forceinline__ static void issue_all(const LoadJob& j) {
 #pragma unroll
@@ -366,6 +378,9 @@ struct AttnWave {
             // operand fetch for group i + PD (of this step, or of the next one)
             if (i + PD < NG) fetch_group(i + PD, kpart1, vpart0, fa[i + PD], fb[i + PD]);
             else fetch_group(i + PD - NG, kpart2, vpart1, pre_a[i + PD - NG], pre_b[i + PD - NG]);
+            // one wait for both fragments of group i (everything but the 2 PD fetches issued since has returned)
+            // instead of one per fragment: every instruction, waits included, costs this wavefront an issue slot
+            if (FULL) __builtin_amdgcn_s_waitcnt(0xC07F | ((2 * PD) << 8));
             if (i < NC) {
                 // ---- stage A, d chunk c = i: S^T, dS^T of tile u+1; softmax of elements [0, 8) ----
                 const int c = i, e0 = c * 8 / NC, e1 = (c + 1) * 8 / NC;
@@ -479,23 +494,23 @@ attn_fwd_jvp_kernel(const AttnParams p) {
         t = t >= n_sweep ? t - n_sweep : t;
         return t >= n_sweep ? t % n_sweep : t;   // (only sweeps shorter than the prefetch depth get here)
     };
-    auto make_job = [&](int u) {
-        const int tk = __builtin_amdgcn_readfirstlane(tile_at(u + 1)), tv = __builtin_amdgcn_readfirstlane(tile_at(u));
+    // tk / tv: tiles whose K part / V part the group copies; ku / vu: sweep positions that pick the ring slots
+    auto make_job = [&](int tk, int ku, int tv, int vu) {
         typename W::LoadJob j;
-        j.rsrc = kv_rsrc; j.lane_off = lane * 16; j.wave = wave;
-        j.k_src = tk * TILE_BYTES; j.k_dst = kring + ((u + 1) % NBUF) * KP_BYTES;
-        j.v_src = tv * TILE_BYTES + KP_BYTES; j.v_dst = vring + (u % NBUF) * VP_BYTES;
+        j.rsrc = kv_rsrc; j.lane_off = lane * 16;
+        j.k_src = tk * TILE_BYTES + W::k_run(wave); j.k_dst = kring + (ku % NBUF) * KP_BYTES + W::k_run(wave);
+        j.v_src = tv * TILE_BYTES + KP_BYTES + W::v_run(wave); j.v_dst = vring + (vu % NBUF) * VP_BYTES + W::v_run(wave);
         return j;
     };
+    auto group_job = [&](int u) { return make_job(tile_at(u + 1), u + 1, tile_at(u), u); };
     {   // K part of the first tile of the sweep (as the K half of a pseudo group "-1"), then groups 0..2
-        typename W::LoadJob j = make_job(0);
-        j.k_src = tile_at(0) * TILE_BYTES; j.k_dst = kring;
+        const typename W::LoadJob j = make_job(tile_at(0), 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < W::KP_LOADS; ++i) W::issue_load(j, i);
     }
-    W::issue_all(make_job(0));
-    W::issue_all(make_job(1));
-    W::issue_all(make_job(2));
+    W::issue_all(group_job(0));
+    W::issue_all(group_job(1));
+    W::issue_all(group_job(2));
 
     W w;
     w.lane = lane;
@@ -541,18 +556,27 @@ attn_fwd_jvp_kernel(const AttnParams p) {
     for (int i = 0; i < W::PD; ++i) w.fetch_group(i, kring + KP_BYTES, vring, w.pre_a[i], w.pre_b[i]);
 
     // Step u: K parts of tiles u+1, u+2 and V parts of tiles u, u+1 are resident (groups u, u+1); group u+2 is in
-    // flight; group u+3 is issued during the step.
+    // flight; group u+3 is issued during the step.  The tiles at sweep positions u+1 (mask test), u+3 and u+4
+    // (fills) are carried as wrapping counters.
+    auto wrap_inc = [&](int t) { ++t; return t >= n_sweep ? t - n_sweep : t; };
+    int t_next = __builtin_amdgcn_readfirstlane(tile_at(1)), t_v = __builtin_amdgcn_readfirstlane(tile_at(3)),
+        t_k = __builtin_amdgcn_readfirstlane(tile_at(4));
     for (int u = 0; u < n_tiles; ++u) {
-        __builtin_amdgcn_s_waitcnt(WAIT_1_GROUP);    // group u+1 landed (this wavefront's share)
-        __syncthreads();                             // ... everyone's share did, and everyone finished step u-1
-        // group u+3 overwrites the K part of tile u and the V part of tile u-1, both dead since the barrier
+        // Group u+1 landed (this wavefront's share) ... then everyone's share did, and everyone finished step u-1.
+        // A bare s_barrier, not __syncthreads(): the fence of the latter would also drain this wavefront's LDS
+        // operand prefetches (lgkmcnt(0)).  None is needed: the fills are tracked by vmcnt, and every LDS read of the
+        // buffers that group u+3 overwrites (K part of tile u, V part of tile u-1) was consumed by an MFMA before
+        // this point.
+        __builtin_amdgcn_s_waitcnt(WAIT_1_GROUP);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
         float mx = w.step(sc, kring + ((u + 1) % NBUF) * KP_BYTES, vring + (u % NBUF) * VP_BYTES,
-                          kring + ((u + 2) % NBUF) * KP_BYTES, vring + ((u + 1) % NBUF) * VP_BYTES, make_job(u + 3));
+                          kring + ((u + 2) % NBUF) * KP_BYTES, vring + ((u + 1) % NBUF) * VP_BYTES, make_job(t_k, u + 4, t_v, u + 3));
         if (u + 1 < n_tiles) {
-            const int tn = tile_at(u + 1);
-            if (need_mask(tn)) mx = W::mask_scores(sc, tn * kBlockN + 4 * hh, kv_len, causal, row);
+            if (need_mask(t_next)) mx = W::mask_scores(sc, t_next * kBlockN + 4 * hh, kv_len, causal, row);
             w.update_max(mx);
         }
+        t_next = wrap_inc(t_next); t_v = wrap_inc(t_v); t_k = wrap_inc(t_k);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // drain the (unused) trailing loads before the LDS is released
 
