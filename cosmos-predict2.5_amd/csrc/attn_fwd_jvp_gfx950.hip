@@ -64,7 +64,7 @@ __device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
 
 constexpr int kBlockM = 128;       // query rows per workgroup (4 wavefronts x 32)
 constexpr int kBlockN = 32;        // keys per tile
-constexpr int kThreads = 256;
+constexpr int kPackThreads = 256;
 constexpr int kFragBytes = 1024;   // one MFMA A-operand fragment: 64 lanes x 16 B
 #ifndef COSMOS_ATTN_PREFETCH_GROUPS
 #define COSMOS_ATTN_PREFETCH_GROUPS 2
@@ -99,7 +99,7 @@ struct PackParams {
 };
 
 // grid (ceil(n_tiles / 2), B*H); every 16-byte unit of a tile image is produced by one thread.
-__global__ void __launch_bounds__(kThreads) pack_kv_kernel(const PackParams p) {
+__global__ void __launch_bounds__(kPackThreads) pack_kv_kernel(const PackParams p) {
     const int bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
     const bool full = p.tk != nullptr;
     const TileGeom g(p.dqk, p.dv, full);
@@ -110,7 +110,7 @@ __global__ void __launch_bounds__(kThreads) pack_kv_kernel(const PackParams p) {
         const int t = blockIdx.x * 2 + tt;
         if (t >= p.n_tiles) break;
         uint4* dst = p.out + ((size_t)bh * p.n_tiles + t) * (size_t)(g.tile_frags * (kFragBytes / 16));
-        for (int u = threadIdx.x; u < units; u += kThreads) {
+        for (int u = threadIdx.x; u < units; u += kPackThreads) {
             int frag = u >> 6;
             const int l = u & 63, i = l & 31, hh = l >> 5;
             uint4 val = make_uint4(0u, 0u, 0u, 0u);
@@ -155,10 +155,13 @@ extern __shared__ __attribute__((aligned(1024))) char smem[];
 
 #define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-// Per-wavefront state and the per-tile work, templated so that everything unrolls into registers.
-template <typename T, int DQK, int DV, int MODE>
-struct AttnWave {
-    typedef typename VecOf<T>::v8 V8;
+constexpr int kAttnThreads = 512;   // 4 score wavefronts + 4 output wavefronts, two per SIMD
+constexpr int kRingK = 4;           // LDS ring depth, K parts
+constexpr int kRingV = 3;           // LDS ring depth, V parts
+
+// Compile-time geometry shared by both roles and the host.
+template <int DQK, int DV, int MODE>
+struct AttnCfg {
     static constexpr int NC = DQK / 16;             // 16-wide d chunks of the QK^T contraction
     static constexpr int NDB = (DV + 31) / 32;      // 32-row blocks of O^T
     static constexpr bool JVP = MODE != MODE_FWD, FULL = MODE == MODE_JVP_FULL;
@@ -168,64 +171,65 @@ struct AttnWave {
     static constexpr int TILE_BYTES = KP_BYTES + VP_BYTES;
     static constexpr int DK_OFF = K_FR * kFragBytes;     // inside the K part
     static constexpr int DVT_OFF = VT_FR * kFragBytes;   // inside the V part
-    static constexpr int KP_LOADS = (KP_FR + 3) / 4, VP_LOADS = (VP_FR + 3) / 4;   // per wavefront per tile
+    static constexpr int KP_LOADS = (KP_FR + 7) / 8, VP_LOADS = (VP_FR + 7) / 8;   // per wavefront per tile (8 wavefronts)
     static constexpr int GROUP_LOADS = KP_LOADS + VP_LOADS;
     static constexpr int MFMA_PER_C = FULL ? 3 : (JVP ? 2 : 1);
-    static constexpr int SLOTS = NC * MFMA_PER_C;        // MFMA issue slots of the score stage
+    // P^T (and H^T) of one tile as MFMA B operands: 2 (4) fragments per score wavefront, double-buffered
+    static constexpr int PH_FR = JVP ? 4 : 2;
+    static constexpr int PH_BYTES = PH_FR * kFragBytes;
+    static constexpr int KRING_OFF = 0;
+    static constexpr int VRING_OFF = kRingK * KP_BYTES;
+    static constexpr int PH_OFF = VRING_OFF + kRingV * VP_BYTES;
+    static constexpr int ALPHA_OFF = PH_OFF + 2 * 4 * PH_BYTES;      // [2 stages][4 wavefronts][64 lanes] floats
+    static constexpr int LDS_BYTES = ALPHA_OFF + 2 * 4 * 256;
+};
+
+// What one wavefront copies per step (one "load group"): its share of the V part of one tile and of the K part
+// of another, as VP_LOADS + KP_LOADS wavefront-level direct-to-LDS loads.  buffer_load ... lds (MUBUF) rather than
+// global_load_lds: the compiler's wait-count pass treats the latter as a FLAT access that may touch LDS and then
+// turns every later LDS wait into lgkmcnt(0).  One wavefront-level load moves one fragment: lane l's 16 bytes
+// (voffset = 16 l) land at dst + 16 l.  The share is a contiguous run of fragments (parts with fewer fragments
+// than wavefronts are copied redundantly), so one LDS base (M0) and one scalar offset serve the whole run and the
+// fragment index travels in the instruction's immediate offset, which is added to both addresses.
+struct LoadJob {
+    __amdgpu_buffer_rsrc_t rsrc;
+    int lane_off;            // 16 * lane
+    int k_src, v_src;        // byte offsets of this wavefront's runs in the packed buffer
+    char *k_dst, *v_dst;     // LDS destinations of the runs
+};
+template <int IMM>
+__device__ __forceinline__ void lds_load(__amdgpu_buffer_rsrc_t rsrc, char* dst, int lane_off, int src) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane_off, src, IMM, 0);
+}
+template <typename C>
+__device__ __forceinline__ void issue_group(const LoadJob& j) {
+    static_assert(C::KP_LOADS <= 2 && C::VP_LOADS <= 2, "a part has at most 16 fragments");
+    lds_load<0>(j.rsrc, j.v_dst, j.lane_off, j.v_src);
+    if (C::VP_LOADS > 1) lds_load<kFragBytes>(j.rsrc, j.v_dst, j.lane_off, j.v_src);
+    lds_load<0>(j.rsrc, j.k_dst, j.lane_off, j.k_src);
+    if (C::KP_LOADS > 1) lds_load<kFragBytes>(j.rsrc, j.k_dst, j.lane_off, j.k_src);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Score wavefront: owns 32 query rows' Q, dQ fragments and softmax statistics.  Per step it issues the score
+// MFMAs of the NEXT tile interleaved with the softmax VALU work of the current one, and hands P^T, H^T (16-bit
+// MFMA B operands) and the rescale factor of the tile to its output wavefront through LDS.
+template <typename T, int DQK, int DV, int MODE>
+struct ScoreWave {
+    typedef AttnCfg<DQK, DV, MODE> C;
+    typedef typename VecOf<T>::v8 V8;
+    static constexpr int NC = C::NC;
+    static constexpr bool JVP = C::JVP, FULL = C::FULL;
+    static constexpr int PD = COSMOS_ATTN_PREFETCH_GROUPS;   // LDS operand fetches run this many chunks ahead of use
 
     // Scores of one tile as this lane sees them: its query column x 16 of the tile's 32 keys (element e is key
-    // 8 (e/4) + 4 (lane/32) + e%4 of the tile).  Kept as plain floats (VGPRs) between steps; the MFMA
-    // accumulators they are copied from live in AccVGPRs only inside a step.
+    // 8 (e/4) + 4 (lane/32) + e%4 of the tile).
     struct Scores { float s[16]; float ds[16]; };
 
-    V8 qf[NC], tqf[NC];                 // (arrays of unused modes are never touched and cost no registers)
-    f32x16 acc[NDB], acct[NDB];
-    static constexpr int PD = COSMOS_ATTN_PREFETCH_GROUPS;   // LDS operand fetches run this many MFMA groups ahead of use
-    V8 pre_a[PD], pre_b[PD];   // LDS fragments of the next step's first PD MFMA groups (fetched ahead)
+    V8 qf[NC], tqf[NC];
     float m_run, l_run, r_run;
     float scale_log2, sm_scale;
     int lane;
-
-    // Direct-to-LDS copy of a part (NFR fragments of 1 KB), spread over the 4 wavefronts; every wavefront issues
-    // the same number of loads (surplus ones repeat a fragment) so that vmcnt bookkeeping is uniform.
-    // buffer_load ... lds (MUBUF) rather than global_load_lds: the compiler's wait-count pass treats the latter as
-    // a FLAT access that may touch LDS and then turns every later LDS wait into lgkmcnt(0), which exposes the
-    // full LDS latency of the operand prefetches.  One wavefront-level load moves one fragment: lane l's 16
-    // bytes (voffset = 16 l) land at dst + 16 l.
-    // What one wavefront copies per step (one "load group"): its share of the K part of one tile and of the V part
-    // of another, as KP_LOADS + VP_LOADS wavefront-level loads.  The share is a contiguous run of fragments
-    // (fragments wave * LOADS .. + LOADS - 1; parts of fewer than 4 fragments are copied redundantly), so one LDS
-    // base (M0) and one scalar offset serve the whole run and the fragment index travels in the instruction's
-    // immediate offset, which is added to both the memory address and the LDS address.
-    struct LoadJob {
-        __amdgpu_buffer_rsrc_t rsrc;
-        int lane_off;            // 16 * lane
-        int k_src, v_src;        // byte offsets of this wavefront's runs in the packed buffer
-        char *k_dst, *v_dst;     // LDS destinations of the runs
-    };
-    __device__ __forceinline__ static int k_run(int wave) { return ((wave * KP_LOADS) % KP_FR) * kFragBytes; }
-    __device__ __forceinline__ static int v_run(int wave) { return ((wave * VP_LOADS) % VP_FR) * kFragBytes; }
-    template <int IMM>
-    __device__ __forceinline__ static void lds_load(__amdgpu_buffer_rsrc_t rsrc, char* dst, int lane_off, int src) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane_off, src, IMM, 0);
-    }
-    // load number i of the group, 0 <= i < GROUP_LOADS (i is a compile-time constant after unrolling; at most 4
-    // loads per part: a part has at most 16 fragments)
-    __device__ __forceinline__ static void issue_load(const LoadJob& j, int i) {
-        const bool kpart = i < KP_LOADS;
-        char* dst = kpart ? j.k_dst : j.v_dst;
-        const int src = kpart ? j.k_src : j.v_src;
-        switch (kpart ? i : i - KP_LOADS) {
-            case 0: lds_load<0>(j.rsrc, dst, j.lane_off, src); break;
-            case 1: lds_load<1 * kFragBytes>(j.rsrc, dst, j.lane_off, src); break;
-            case 2: lds_load<2 * kFragBytes>(j.rsrc, dst, j.lane_off, src); break;
-            default: lds_load<3 * kFragBytes>(j.rsrc, dst, j.lane_off, src); break;
-        }
-    }
-    __device__ __forceinline__ static void issue_all(const LoadJob& j) {
-#pragma unroll
-        for (int i = 0; i < GROUP_LOADS; ++i) issue_load(j, i);
-    }
 
     __device__ __forceinline__ V8 lds_frag(const char* base, int frag) const {
         return *reinterpret_cast<const V8*>(base + frag * kFragBytes + lane * 16);
@@ -245,7 +249,96 @@ struct AttnWave {
         return mx;
     }
 
-    // scores of one tile with nothing interleaved (prologue); returns the lane-local max of s
+    // Fold a tile's lane-local score max into the running max.  Returns the factor by which everything accumulated
+    // so far must be rescaled before this tile is added (exactly 1 when no row's max moved).
+    __device__ __forceinline__ float update_max(float mx) {
+        {   // max with lane ^ 32 (the other half of the same query column): one VALU swap, no LDS round trip
+            const unsigned bits = __builtin_bit_cast(unsigned, mx);
+            const auto sw = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+            mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+        }
+        const float m_new = fmaxf(m_run, mx * scale_log2);
+        float alpha = 1.0f;
+        if (__any(m_new > m_run)) {
+            alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= alpha;
+            r_run *= alpha;
+            m_run = m_new;
+        }
+        return alpha;
+    }
+
+    // Softmax of element e of this lane's 16:  p = exp2(s c - m), l += p ;  H = p dS s, r += H.  Both rounded to
+    // 16-bit MFMA operands.
+    __device__ __forceinline__ void softmax_elem(const Scores& x, V8* pf, V8* hf, int e) {
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(x.s[e], scale_log2, -m_run));
+        l_run += p;
+        pf[e >> 3][e & 7] = (T)p;
+        if (JVP) {
+            const float hv = p * (x.ds[e] * sm_scale);
+            r_run += hv;
+            hf[e >> 3][e & 7] = (T)hv;
+        }
+    }
+
+    // One step: softmax of the tile whose scores are in `x` (already folded into m_run) and, if `next`, the scores
+    // of the next tile from `kpart` into `x`.  P^T / H^T go to `ph_out`, `alpha` to `alpha_out`.
+    // Returns the lane-local max of the new scores.
+    __device__ __forceinline__ float step(Scores& x, const char* kpart, unsigned ph_out, unsigned alpha_out, float alpha) {
+        V8 pf[2], hf[2];
+        V8 fa[NC], fb[NC];
+        asm volatile("ds_write_b32 %0, %1" ::"v"(alpha_out + 4 * lane), "v"(alpha) : "memory");
+#pragma unroll
+        for (int i = 0; i < PD && i < NC; ++i) { fa[i] = lds_frag(kpart, i); if (FULL) fb[i] = lds_frag(kpart + C::DK_OFF, i); }
+        f32x16 sn, dsn;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { sn[e] = 0.f; dsn[e] = 0.f; }
+        constexpr int EPC = 16 / NC;   // softmax elements dealt out per chunk (NC <= 8)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            SCHED_FENCE();
+            if (c + PD < NC) { fa[c + PD] = lds_frag(kpart, c + PD); if (FULL) fb[c + PD] = lds_frag(kpart + C::DK_OFF, c + PD); }
+            SCHED_FENCE();
+            sn = mfma32(fa[c], qf[c], sn);
+#pragma unroll
+            for (int k = 0; k < EPC; ++k)
+                if (k * C::MFMA_PER_C / EPC == 0) softmax_elem(x, pf, hf, c * EPC + k);
+            SCHED_FENCE();
+            if (JVP) {
+                dsn = mfma32(fa[c], tqf[c], dsn);
+#pragma unroll
+                for (int k = 0; k < EPC; ++k)
+                    if (k * C::MFMA_PER_C / EPC == 1) softmax_elem(x, pf, hf, c * EPC + k);
+                SCHED_FENCE();
+            }
+            if (FULL) {
+                dsn = mfma32(fb[c], qf[c], dsn);
+#pragma unroll
+                for (int k = 0; k < EPC; ++k)
+                    if (k * C::MFMA_PER_C / EPC == 2) softmax_elem(x, pf, hf, c * EPC + k);
+                SCHED_FENCE();
+            }
+        }
+        // hand P^T, H^T over (asm stores: a visible LDS store would make the compiler wait for vmcnt(0), i.e. for
+        // the direct-to-LDS fills in flight)
+        const unsigned pa = ph_out + 16 * lane;
+        asm volatile("ds_write_b128 %0, %1" ::"v"(pa), "v"(pf[0]) : "memory");
+        asm volatile("ds_write_b128 %0, %1 offset:1024" ::"v"(pa), "v"(pf[1]) : "memory");
+        if (JVP) {
+            asm volatile("ds_write_b128 %0, %1 offset:2048" ::"v"(pa), "v"(hf[0]) : "memory");
+            asm volatile("ds_write_b128 %0, %1 offset:3072" ::"v"(pa), "v"(hf[1]) : "memory");
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            x.s[e] = sn[e];
+            if (JVP) x.ds[e] = dsn[e];
+            mx = fmaxf(mx, x.s[e]);
+        }
+        return mx;
+    }
+
+    // scores of the first tile (prologue); returns the lane-local max
     __device__ __forceinline__ float scores_plain(Scores& x, const char* kpart) const {
         f32x16 s, ds;
 #pragma unroll
@@ -255,213 +348,97 @@ struct AttnWave {
             const V8 kf = lds_frag(kpart, c);
             if (JVP) ds = mfma32(kf, tqf[c], ds);
             s = mfma32(kf, qf[c], s);
-            if (FULL) ds = mfma32(lds_frag(kpart + DK_OFF, c), qf[c], ds);
+            if (FULL) ds = mfma32(lds_frag(kpart + C::DK_OFF, c), qf[c], ds);
         }
-        // explicit AccVGPR -> VGPR copies (as in step(), so that the scores carried between steps are VGPR values
-        // for every definition); the wait states after the last MFMA are spelled out
-        // (inside the same asm statements as the reads: a separate nop statement could be scheduled away from them)
         float mx = -INFINITY;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            float sv = s[e];
-            asm volatile("s_nop 15\n\ts_nop 7\n\tv_accvgpr_read_b32 %0, %1" : "=v"(x.s[e]) : "a"(sv));
-            if (JVP) {
-                float dv = ds[e];
-                asm volatile("s_nop 15\n\ts_nop 7\n\tv_accvgpr_read_b32 %0, %1" : "=v"(x.ds[e]) : "a"(dv));
-            }
+            x.s[e] = s[e];
+            if (JVP) x.ds[e] = ds[e];
             mx = fmaxf(mx, x.s[e]);
         }
         return mx;
     }
+};
 
-    // Softmax of element e of this lane's 16, in two halves so that the VALU work can be spread thinly between
-    // MFMAs:  p = exp2(s c - m), l += p   and   H = p dS s, r += H.   Both are rounded to 16-bit MFMA operands.
-    __device__ __forceinline__ void softmax_p(const Scores& x, float* pv, V8* pf, int e) {
-        pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(x.s[e], scale_log2, -m_run));
-        l_run += pv[e];
-        pf[e >> 3][e & 7] = (T)pv[e];
+// ---------------------------------------------------------------------------------------------------------------
+// Output wavefront: owns the fp32 accumulators O^T and T^T (= (P dV + H V)^T; the reference keeps the two terms
+// apart, JVP:134-146, but only ever uses their sum, JVP:369) of the same 32 query rows.
+template <typename T, int DQK, int DV, int MODE>
+struct OutputWave {
+    typedef AttnCfg<DQK, DV, MODE> C;
+    typedef typename VecOf<T>::v8 V8;
+    static constexpr int NDB = C::NDB;
+    static constexpr bool JVP = C::JVP, FULL = C::FULL;
+    static constexpr int NB = 2 * NDB;      // MFMA groups of a step, g = c * NDB + db
+    static constexpr int PD = COSMOS_ATTN_PREFETCH_GROUPS;
+
+    f32x16 acc[NDB], acct[NDB];
+    int lane;
+
+    __device__ __forceinline__ V8 lds_frag(const char* base, int frag) const {
+        return *reinterpret_cast<const V8*>(base + frag * kFragBytes + lane * 16);
     }
-    __device__ __forceinline__ void softmax_h(const Scores& x, const float* pv, V8* hf, int e) {
-        if (JVP) {
-            const float hv = pv[e] * (x.ds[e] * sm_scale);
-            r_run += hv;
-            hf[e >> 3][e & 7] = (T)hv;
-        }
+    __device__ __forceinline__ void fetch_group(int g, const char* vpart, V8& a, V8& b) const {
+        const int c = g / NDB, db = g % NDB;
+        a = lds_frag(vpart, 2 * db + c);
+        if (FULL) b = lds_frag(vpart + C::DVT_OFF, 2 * db + c);
     }
 
-    // Fold a tile's lane-local score max into the running max; rescale the accumulators when some row's max
-    // moved (wavefront-uniform branch; alpha == 1 exactly otherwise).
-    __device__ __forceinline__ void update_max(float mx) {
-        {   // max with lane ^ 32 (the other half of the same query column): one VALU swap, no LDS round trip
-            const unsigned bits = __builtin_bit_cast(unsigned, mx);
-            const auto sw = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
-            mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
-        }
-        const float m_new = fmaxf(m_run, mx * scale_log2);
-        if (__any(m_new > m_run)) {
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-            l_run *= alpha;
-            r_run *= alpha;
-            // The accumulators live in AccVGPRs for the whole KV sweep (they are only ever MFMA operands).  This
-            // rare path scales them in place through a scratch VGPR; the "+a" constraints keep the register
-            // allocator from copying all of them to VGPRs around the branch on every step.  The MFMA -> AccVGPR
-            // read and AccVGPR write -> MFMA dependencies are invisible to the compiler inside the asm, so the
-            // required wait states are spelled out as s_nop.
+    // One step: O^T = alpha O^T + V^T P^T ;  T^T = alpha T^T + V^T H^T + dV^T P^T
+    __device__ __forceinline__ void step(const char* vpart, const char* ph_in, const char* alpha_in) {
+        const float alpha = *reinterpret_cast<const float*>(alpha_in + 4 * lane);
+        V8 pf[2], hf[2];
+        pf[0] = lds_frag(ph_in, 0); pf[1] = lds_frag(ph_in, 1);
+        if (JVP) { hf[0] = lds_frag(ph_in, 2); hf[1] = lds_frag(ph_in, 3); }
+        V8 fa[NB], fb[NB];
+#pragma unroll
+        for (int i = 0; i < PD && i < NB; ++i) fetch_group(i, vpart, fa[i], fb[i]);
+        if (__any(alpha != 1.0f)) {   // some row's max moved (wavefront-uniform, rare after the first tiles)
 #pragma unroll
             for (int i = 0; i < NDB; ++i) {
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    // the first statement of each accumulator carries the MFMA -> read wait states
-                    float x = acc[i][e], tmp;
-                    if (e == 0)
-                        asm volatile("s_nop 15\n\ts_nop 7\n\tv_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 3"
-                                     : "+a"(x), "=&v"(tmp) : "v"(alpha));
-                    else
-                        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 3"
-                                     : "+a"(x), "=&v"(tmp) : "v"(alpha));
-                    acc[i][e] = x;
-                    if (JVP) {
-                        float y = acct[i][e], tmp2;
-                        if (e == 0)
-                            asm volatile("s_nop 15\n\ts_nop 7\n\tv_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 3"
-                                         : "+a"(y), "=&v"(tmp2) : "v"(alpha));
-                        else
-                            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 3"
-                                         : "+a"(y), "=&v"(tmp2) : "v"(alpha));
-                        acct[i][e] = y;
-                    }
-                }
+                for (int e = 0; e < 16; ++e) { acc[i][e] *= alpha; if (JVP) acct[i][e] *= alpha; }
             }
-            m_run = m_new;
         }
-    }
-
-    static constexpr int NB = 2 * NDB;      // MFMA groups of stage B, g = c * NDB + db
-    static constexpr int NG = NC + NB;      // MFMA groups of a step: stage A chunk c = i, then stage B group g = i - NC
-
-    // LDS fragments of MFMA group i of a step whose stage A reads `kpart` and whose stage B reads `vpart`
-    __device__ __forceinline__ void fetch_group(int i, const char* kpart, const char* vpart, V8& a, V8& b) const {
-        if (i < NC) {
-            a = lds_frag(kpart, i);
-            if (FULL) b = lds_frag(kpart + DK_OFF, i);
-        } else {
-            const int g = i - NC, c = g / NDB, db = g % NDB;
-            a = lds_frag(vpart, 2 * db + c);
-            if (FULL) b = lds_frag(vpart + DVT_OFF, 2 * db + c);
-        }
-    }
-
-    // One software-pipelined step over tile u (scores in `x`, already folded into m_run):
-    //   stage A: scores of tile u+1 (MFMA) | softmax of the first 8 keys per lane (VALU) | this step's LDS fills;
-    //   stage B, first half:  P.V-type products over those keys (MFMA) | softmax of the other 8 keys (VALU);
-    //   stage B, second half: products over the other keys (MFMA) | copy-out of the new scores to VGPRs.
-    // On return `x` holds the scores of tile u+1; the return value is their lane-local max.
-    // kpart1 / vpart0: K part of tile u+1, V part of tile u (this step); kpart2 / vpart1: those of the next step,
-    // already resident, from which the last PD groups fetch the next step's first fragments -- the stream of LDS
-    // operand fetches (PD groups ahead of use) never drains, not even across the workgroup barrier.
-    // A wavefront hides roughly 5 VALU instructions behind one 8-pass MFMA, so the VALU work is dealt out in
-    // slices of that size; scheduling fences keep the written interleaving.
-    __device__ __forceinline__ float step(Scores& x, const char* kpart1, const char* vpart0, const char* kpart2, const char* vpart1,
-                                          const LoadJob& job) {
-        V8 pf[2], hf[2];
-        float pv[16];
-        V8 fa[NG], fb[NG];
 #pragma unroll
-        for (int i = 0; i < PD; ++i) { fa[i] = pre_a[i]; if (FULL) fb[i] = pre_b[i]; }
-        f32x16 sn, dsn;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) { sn[e] = 0.f; dsn[e] = 0.f; }
-        float mx = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < NG; ++i) {
+        for (int g = 0; g < NB; ++g) {
+            const int c = g / NDB, db = g % NDB;
             SCHED_FENCE();
-            // operand fetch for group i + PD (of this step, or of the next one)
-            if (i + PD < NG) fetch_group(i + PD, kpart1, vpart0, fa[i + PD], fb[i + PD]);
-            else fetch_group(i + PD - NG, kpart2, vpart1, pre_a[i + PD - NG], pre_b[i + PD - NG]);
-            // one wait for both fragments of group i (everything but the 2 PD fetches issued since has returned)
-            // instead of one per fragment: every instruction, waits included, costs this wavefront an issue slot
-            if (FULL) __builtin_amdgcn_s_waitcnt(0xC07F | ((2 * PD) << 8));
-            if (i < NC) {
-                // ---- stage A, d chunk c = i: S^T, dS^T of tile u+1; softmax of elements [0, 8) ----
-                const int c = i, e0 = c * 8 / NC, e1 = (c + 1) * 8 / NC;
-#pragma unroll
-                for (int k = c * GROUP_LOADS / NC; k < (c + 1) * GROUP_LOADS / NC; ++k) issue_load(job, k);
-                SCHED_FENCE();
-                sn = mfma32(fa[i], qf[c], sn);
-#pragma unroll
-                for (int e = e0; e < e1; ++e) softmax_p(x, pv, pf, e);
-                SCHED_FENCE();
-                if (JVP) {
-                    dsn = mfma32(fa[i], tqf[c], dsn);
-#pragma unroll
-                    for (int e = e0; e < e1; ++e) softmax_h(x, pv, hf, e);
-                    SCHED_FENCE();
-                }
-                if (FULL) dsn = mfma32(fb[i], qf[c], dsn);
-            } else {
-                // ---- stage B, group g: O^T += V^T P^T ; T^T += V^T H^T + dV^T P^T ----
-                const int g = i - NC, c = g / NDB, db = g % NDB;
-                SCHED_FENCE();
-                acc[db] = mfma32(fa[i], pf[c], acc[db]);
-                if (c == 0) {   // first half: softmax of elements [8, 16), p-halves
-#pragma unroll
-                    for (int e = 8 + db * 8 / NDB; e < 8 + (db + 1) * 8 / NDB; ++e) softmax_p(x, pv, pf, e);
-                }
-                SCHED_FENCE();
-                if (JVP) acct[db] = mfma32(fa[i], hf[c], acct[db]);
-                if (c == 0) {   // ... h-halves
-#pragma unroll
-                    for (int e = 8 + db * 8 / NDB; e < 8 + (db + 1) * 8 / NDB; ++e) softmax_h(x, pv, hf, e);
-                }
-                if (JVP) SCHED_FENCE();
-                if (FULL) acct[db] = mfma32(fb[i], pf[c], acct[db]);
-                if (c == 1) {
-                    // Second half: copy-out of the next tile's scores (AccVGPR -> VGPR), a slice per group.  Explicit
-                    // instructions: the copy must happen HERE (in the shadow of the MFMA pipe), not wherever the
-                    // register allocator would otherwise place it.  The hardware does not interlock an AccVGPR read
-                    // against the MFMA that produces the register and the compiler cannot see inside the asm; the
-                    // scores were last written in stage A, NDB full MFMA groups before the first read (plus explicit
-                    // wait states), which exceeds the 8-pass MFMA -> read requirement.
-#pragma unroll
-                    for (int e = db * 16 / NDB; e < (db + 1) * 16 / NDB; ++e) {
-                        float sv = sn[e];
-                        if (e == 0 && NDB * MFMA_PER_C >= 6) asm volatile("s_nop 3\n\tv_accvgpr_read_b32 %0, %1" : "=v"(x.s[e]) : "a"(sv));
-                        else if (e == 0) asm volatile("s_nop 15\n\ts_nop 3\n\tv_accvgpr_read_b32 %0, %1" : "=v"(x.s[e]) : "a"(sv));
-                        else asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x.s[e]) : "a"(sv));
-                        if (JVP) {
-                            float dv = dsn[e];
-                            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x.ds[e]) : "a"(dv));
-                        }
-                        mx = fmaxf(mx, x.s[e]);
-                    }
-                }
-            }
+            if (g + PD < NB) fetch_group(g + PD, vpart, fa[g + PD], fb[g + PD]);
+            SCHED_FENCE();
+            acc[db] = mfma32(fa[g], pf[c], acc[db]);
+            if (JVP) acct[db] = mfma32(fa[g], hf[c], acct[db]);
+            if (FULL) acct[db] = mfma32(fb[g], pf[c], acct[db]);
         }
         SCHED_FENCE();
-        return mx;
     }
 };
 
 template <typename T, int DQK, int DV, int MODE>
-__global__ void __attribute__((amdgpu_flat_work_group_size(kThreads, kThreads), amdgpu_waves_per_eu(1, 1)))
+__global__ void __attribute__((amdgpu_flat_work_group_size(kAttnThreads, kAttnThreads), amdgpu_waves_per_eu(2, 2)))
 attn_fwd_jvp_kernel(const AttnParams p) {
-    typedef AttnWave<T, DQK, DV, MODE> W;
-    typedef typename W::V8 V8;
+    typedef AttnCfg<DQK, DV, MODE> C;
+    typedef ScoreWave<T, DQK, DV, MODE> SW;
+    typedef OutputWave<T, DQK, DV, MODE> OW;
+    typedef typename VecOf<T>::v8 V8;
     typedef typename VecOf<T>::v4 V4;
-    constexpr int NC = W::NC, NDB = W::NDB;
-    constexpr bool JVP = W::JVP;
-    constexpr int KP_BYTES = W::KP_BYTES, VP_BYTES = W::VP_BYTES, TILE_BYTES = W::TILE_BYTES;
-    constexpr int NBUF = 4;                              // LDS ring depth for K parts and for V parts
-    constexpr int GROUP_LOADS = W::GROUP_LOADS;   // loads per wavefront in one load group
-    // s_waitcnt immediates: vmcnt(n) with expcnt / lgkmcnt left at their maxima
-    constexpr int WAIT_1_GROUP = (GROUP_LOADS & 15) | ((GROUP_LOADS >> 4) << 14) | 0x0F70;
-    static_assert(3 * GROUP_LOADS + W::KP_LOADS <= 63, "vmcnt range");
+    constexpr int NC = C::NC, NDB = C::NDB;
+    constexpr bool JVP = C::JVP;
+    constexpr int KP_BYTES = C::KP_BYTES, VP_BYTES = C::VP_BYTES, TILE_BYTES = C::TILE_BYTES;
+    // s_waitcnt immediate: vmcnt(n), expcnt / lgkmcnt left at their maxima.  At the top of step s the fills of the
+    // V part of tile s-1 and the K part of tile s+1 must have landed; issued after them (in this order) and still
+    // allowed in flight: K(s+2), V(s), K(s+3).
+    constexpr int IN_FLIGHT = 2 * C::KP_LOADS + C::VP_LOADS;
+    constexpr int WAIT_FILLS = (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14) | 0x0F70;
 
     const int qt = blockIdx.x, bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const bool score_role = wave < 4;            // wavefronts w and w + 4 (same SIMD) serve query rows 32 w .. 32 w + 31
+    const int qw = wave & 3;
     const int j = lane & 31, hh = lane >> 5;
-    const int row0 = qt * kBlockM + wave * 32;   // first query row of this wavefront
+    const int row0 = qt * kBlockM + qw * 32;     // first query row of this wavefront pair
     const int row = row0 + j;                    // this lane's query row (lanes l and l^32 share it)
 
     int kv_len = p.Lkv;
@@ -469,12 +446,8 @@ attn_fwd_jvp_kernel(const AttnParams p) {
     int n_tiles = (kv_len + kBlockN - 1) / kBlockN;
     if (p.causal) { const int lim = (qt * kBlockM + kBlockM + kBlockN - 1) / kBlockN; n_tiles = n_tiles < lim ? n_tiles : lim; }
 
-    // LDS: ring of NBUF K-part buffers, then ring of NBUF V-part buffers.
-    // Load group G(u) = { K part of the tile at sweep position u+1, V part of the tile at position u }: what step u
-    // needs.  Positions past the end wrap around (that data is loaded but never used) so every wavefront always
-    // issues the same number of loads.
-    char* const kring = smem;
-    char* const vring = smem + NBUF * KP_BYTES;
+    char* const kring = smem + C::KRING_OFF;
+    char* const vring = smem + C::VRING_OFF;
     // buffer resource over this (batch, head)'s packed tiles: raw (stride 0), num_records in bytes
     const __amdgpu_buffer_rsrc_t kv_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<char*>(p.kv) + (size_t)bh * p.n_tiles * TILE_BYTES, 0, p.n_tiles * TILE_BYTES, 0x00020000);
@@ -488,126 +461,151 @@ attn_fwd_jvp_kernel(const AttnParams p) {
     // (not with causal masking: there the first tile of the sweep must be tile 0, the one tile in which every query row
     // sees a key, so that the running max is finite from the first step on)
     const int shift = p.causal ? 0 : (((wg_linear >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
-    auto tile_at = [&](int u) {
-        int t = u + shift;
-        t = t >= n_sweep ? t - n_sweep : t;
-        t = t >= n_sweep ? t - n_sweep : t;
-        return t >= n_sweep ? t % n_sweep : t;   // (only sweeps shorter than the prefetch depth get here)
-    };
+    auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane((u + shift) % n_sweep); };
+    auto wrap_inc = [&](int t) { ++t; return t >= n_sweep ? t - n_sweep : t; };
+    const int k_run = ((wave * C::KP_LOADS) % C::KP_FR) * kFragBytes, v_run = ((wave * C::VP_LOADS) % C::VP_FR) * kFragBytes;
     // tk / tv: tiles whose K part / V part the group copies; ku / vu: sweep positions that pick the ring slots
     auto make_job = [&](int tk, int ku, int tv, int vu) {
-        typename W::LoadJob j;
-        j.rsrc = kv_rsrc; j.lane_off = lane * 16;
-        j.k_src = tk * TILE_BYTES + W::k_run(wave); j.k_dst = kring + (ku % NBUF) * KP_BYTES + W::k_run(wave);
-        j.v_src = tv * TILE_BYTES + KP_BYTES + W::v_run(wave); j.v_dst = vring + (vu % NBUF) * VP_BYTES + W::v_run(wave);
-        return j;
+        LoadJob jb;
+        jb.rsrc = kv_rsrc; jb.lane_off = lane * 16;
+        jb.k_src = tk * TILE_BYTES + k_run; jb.k_dst = kring + (ku % kRingK) * KP_BYTES + k_run;
+        jb.v_src = tv * TILE_BYTES + KP_BYTES + v_run; jb.v_dst = vring + (vu % kRingV) * VP_BYTES + v_run;
+        return jb;
     };
-    auto group_job = [&](int u) { return make_job(tile_at(u + 1), u + 1, tile_at(u), u); };
-    {   // K part of the first tile of the sweep (as the K half of a pseudo group "-1"), then groups 0..2
-        const typename W::LoadJob j = make_job(tile_at(0), 0, 0, 0);
+    // Fill stream, in issue order:  K(0) K(1) K(2) [V(0) K(3)] | step 0: [V(1) K(4)] | step 1: [V(2) K(5)] | ...
+    // (positions past the end of the sweep wrap around: that data is loaded but never used, so that every
+    // wavefront always issues the same number of loads)
 #pragma unroll
-        for (int i = 0; i < W::KP_LOADS; ++i) W::issue_load(j, i);
+    for (int u = 0; u < 3; ++u) {
+        const LoadJob jb = make_job(tile_at(u), u, 0, 0);
+        lds_load<0>(jb.rsrc, jb.k_dst, jb.lane_off, jb.k_src);
+        if (C::KP_LOADS > 1) lds_load<kFragBytes>(jb.rsrc, jb.k_dst, jb.lane_off, jb.k_src);
     }
-    W::issue_all(group_job(0));
-    W::issue_all(group_job(1));
-    W::issue_all(group_job(2));
-
-    W w;
-    w.lane = lane;
-    w.scale_log2 = p.scale_log2;
-    w.sm_scale = p.sm_scale;
-    {   // Q (and dQ) fragments: B operand of S^T = K Q^T; lane holds Q[row][16 c + 8 hh .. +7]
-        const int64_t off = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh + (int64_t)row * p.q_sl + 8 * hh;
-        const T* qp = reinterpret_cast<const T*>(p.q) + off;
-        const T* tqp = reinterpret_cast<const T*>(p.tq) + off;
-        const bool live = row < p.Lq;
-#pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            V8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-            w.qf[c] = live ? *reinterpret_cast<const V8*>(qp + 16 * c) : z;
-            if (JVP) w.tqf[c] = live ? *reinterpret_cast<const V8*>(tqp + 16 * c) : z;
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < NDB; ++i) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) { w.acc[i][e] = 0.f; if (JVP) w.acct[i][e] = 0.f; }
-    }
-    w.m_run = -INFINITY;   // running row max of the scaled scores, log2 domain (same in lanes l and l^32)
-    w.l_run = 0.f;         // this lane's partial row sum of p (the two half rows are added in the epilogue)
-    w.r_run = 0.f;         // this lane's partial row sum of H
+    issue_group<C>(make_job(tile_at(3), 3, tile_at(0), 0));
 
     const bool causal = p.causal != 0;
-    // wavefront-uniform: does tile u hold a key some row of this wavefront must not see?
+    // wavefront-uniform: does tile t hold a key some row of this wavefront must not see?
     auto need_mask = [&](int t) { return (t * kBlockN + kBlockN > kv_len) || (causal && (t * kBlockN + kBlockN - 1 > row0)); };
+    // LDS byte offsets (from `smem`) of this wavefront pair's hand-over slots; stage k adds k * 4 * PH_BYTES / k * 4 * 256
+    const unsigned ph_base = C::PH_OFF + qw * C::PH_BYTES, alpha_base = C::ALPHA_OFF + qw * 256;
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;   // LDS address of smem[0], for asm stores
+    int t_v = tile_at(1), t_k = tile_at(4);
 
-    typename W::Scores sc;
-    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): everything issued so far has landed (this wavefront's share)
-    __syncthreads();
-    {
-        float mx = w.scores_plain(sc, kring);
-        const int t0 = tile_at(0);
-        if (need_mask(t0)) mx = W::mask_scores(sc, t0 * kBlockN + 4 * hh, kv_len, causal, row);
-        if (n_tiles > 0) w.update_max(mx);
-    }
-
-    // fragments of step 0's first two MFMA groups
+    if (score_role) {
+        SW w;
+        w.lane = lane;
+        w.scale_log2 = p.scale_log2;
+        w.sm_scale = p.sm_scale;
+        {   // Q (and dQ) fragments: B operand of S^T = K Q^T; lane holds Q[row][16 c + 8 hh .. +7]
+            const int64_t off = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh + (int64_t)row * p.q_sl + 8 * hh;
+            const T* qp = reinterpret_cast<const T*>(p.q) + off;
+            const T* tqp = reinterpret_cast<const T*>(p.tq) + off;
+            const bool live = row < p.Lq;
 #pragma unroll
-    for (int i = 0; i < W::PD; ++i) w.fetch_group(i, kring + KP_BYTES, vring, w.pre_a[i], w.pre_b[i]);
+            for (int c = 0; c < NC; ++c) {
+                V8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+                w.qf[c] = live ? *reinterpret_cast<const V8*>(qp + 16 * c) : z;
+                if (JVP) w.tqf[c] = live ? *reinterpret_cast<const V8*>(tqp + 16 * c) : z;
+            }
+        }
+        w.m_run = -INFINITY;   // running row max of the scaled scores, log2 domain (same in lanes l and l^32)
+        w.l_run = 0.f;         // this lane's partial row sum of p (the two half rows are added in the epilogue)
+        w.r_run = 0.f;         // this lane's partial row sum of H
 
-    // Step u: K parts of tiles u+1, u+2 and V parts of tiles u, u+1 are resident (groups u, u+1); group u+2 is in
-    // flight; group u+3 is issued during the step.  The tiles at sweep positions u+1 (mask test), u+3 and u+4
-    // (fills) are carried as wrapping counters.
-    auto wrap_inc = [&](int t) { ++t; return t >= n_sweep ? t - n_sweep : t; };
-    int t_next = __builtin_amdgcn_readfirstlane(tile_at(1)), t_v = __builtin_amdgcn_readfirstlane(tile_at(3)),
-        t_k = __builtin_amdgcn_readfirstlane(tile_at(4));
-    for (int u = 0; u < n_tiles; ++u) {
-        // Group u+1 landed (this wavefront's share) ... then everyone's share did, and everyone finished step u-1.
-        // A bare s_barrier, not __syncthreads(): the fence of the latter would also drain this wavefront's LDS
-        // operand prefetches (lgkmcnt(0)).  None is needed: the fills are tracked by vmcnt, and every LDS read of the
-        // buffers that group u+3 overwrites (K part of tile u, V part of tile u-1) was consumed by an MFMA before
-        // this point.
-        __builtin_amdgcn_s_waitcnt(WAIT_1_GROUP);
+        typename SW::Scores sc;
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): everything issued so far has landed (this wavefront's share)
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        float mx = w.step(sc, kring + ((u + 1) % NBUF) * KP_BYTES, vring + (u % NBUF) * VP_BYTES,
-                          kring + ((u + 2) % NBUF) * KP_BYTES, vring + ((u + 1) % NBUF) * VP_BYTES, make_job(t_k, u + 4, t_v, u + 3));
-        if (u + 1 < n_tiles) {
-            if (need_mask(t_next)) mx = W::mask_scores(sc, t_next * kBlockN + 4 * hh, kv_len, causal, row);
-            w.update_max(mx);
+        float alpha = 1.0f;
+        {
+            float mx = w.scores_plain(sc, kring);
+            const int t0 = tile_at(0);
+            if (need_mask(t0)) mx = SW::mask_scores(sc, t0 * kBlockN + 4 * hh, kv_len, causal, row);
+            if (n_tiles > 0) alpha = w.update_max(mx);
         }
-        t_next = wrap_inc(t_next); t_v = wrap_inc(t_v); t_k = wrap_inc(t_k);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);   // drain the (unused) trailing loads before the LDS is released
-
-    // ---- epilogue: O = acc / l ; dO = (T - r O) / l ; LSE = (m + log2 l) ln 2 ----
-    const float l_tot = w.l_run + __shfl_xor(w.l_run, 32);
-    const float r_tot = w.r_run + __shfl_xor(w.r_run, 32);
-    const float inv_l = 1.0f / l_tot;
-    const float r_over_l = r_tot * inv_l;
-    if (row < p.Lq) {
-        const int64_t off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)row * p.o_sl;
-        T* op = reinterpret_cast<T*>(p.o) + off;
-        T* top = reinterpret_cast<T*>(p.to) + off;
+        // Step s: softmax of tile s, scores of tile s+1 (K part resident since the barrier at the top of the step).
+        for (int s = 0; s <= n_tiles; ++s) {
+            // own P^T / H^T stores of step s-1 done (lgkmcnt(0)), own fills of V(s-1), K(s+1) landed (vmcnt); the
+            // barrier then says the same of every wavefront, and that every wavefront finished step s-1
+            __builtin_amdgcn_s_waitcnt(WAIT_FILLS & 0xF0FF);
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            // V(s+1) overwrites V(s-2), K(s+4) overwrites K(s): both dead since the barrier
+            issue_group<C>(make_job(t_k, s + 4, t_v, s + 1));
+            if (s < n_tiles) {
+                float mx = w.step(sc, kring + ((s + 1) % kRingK) * KP_BYTES, lds0 + ph_base + (s & 1) * 4 * C::PH_BYTES,
+                                  lds0 + alpha_base + (s & 1) * 4 * 256, alpha);
+                if (s + 1 < n_tiles) {
+                    if (need_mask(t_v)) mx = SW::mask_scores(sc, t_v * kBlockN + 4 * hh, kv_len, causal, row);
+                    alpha = w.update_max(mx);
+                }
+            }
+            t_v = wrap_inc(t_v); t_k = wrap_inc(t_k);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0070);   // drain the (unused) trailing fills and the last stores
+        __builtin_amdgcn_s_barrier();         // the output wavefronts have read the last alpha
+        // ---- epilogue, statistics: 1 / l and r / l to the output wavefront ; LSE = (m + log2 l) ln 2 ----
+        const float l_tot = w.l_run + __shfl_xor(w.l_run, 32);
+        const float r_tot = w.r_run + __shfl_xor(w.r_run, 32);
+        const float inv_l = 1.0f / l_tot;
+        const float r_over_l = r_tot * inv_l;
+        asm volatile("ds_write_b32 %0, %1" ::"v"(lds0 + alpha_base + 4 * lane), "v"(inv_l) : "memory");
+        asm volatile("ds_write_b32 %0, %1" ::"v"(lds0 + alpha_base + 4 * 256 + 4 * lane), "v"(r_over_l) : "memory");
+        __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        if (row < p.Lq && p.lse && hh == 0) p.lse[(int64_t)bh * p.Lq + row] = (w.m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
+    } else {
+        OW w;
+        w.lane = lane;
 #pragma unroll
-        for (int db = 0; db < NDB; ++db) {
+        for (int i = 0; i < NDB; ++i) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int d = 32 * db + 8 * g + 4 * hh;   // registers 4g..4g+3 are 4 consecutive d
-                if (d < DV) {
-                    V4 ov, tov;
+            for (int e = 0; e < 16; ++e) { w.acc[i][e] = 0.f; if (JVP) w.acct[i][e] = 0.f; }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // Step s: accumulate tile s-1 (P^T, H^T, alpha written by the score wavefront during step s-1).
+        for (int s = 0; s <= n_tiles; ++s) {
+            __builtin_amdgcn_s_waitcnt(WAIT_FILLS);
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            issue_group<C>(make_job(t_k, s + 4, t_v, s + 1));
+            if (s > 0)
+                w.step(vring + ((s - 1) % kRingV) * VP_BYTES, smem + ph_base + ((s - 1) & 1) * 4 * C::PH_BYTES,
+                       smem + alpha_base + ((s - 1) & 1) * 4 * 256);
+            t_v = wrap_inc(t_v); t_k = wrap_inc(t_k);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // ---- epilogue, outputs: O = acc / l ; dO = (T - (r / l) acc) / l ----
+        const float inv_l = *reinterpret_cast<const float*>(smem + alpha_base + 4 * lane);
+        const float r_over_l = *reinterpret_cast<const float*>(smem + alpha_base + 4 * 256 + 4 * lane);
+        if (row < p.Lq) {
+            const int64_t off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)row * p.o_sl;
+            T* op = reinterpret_cast<T*>(p.o) + off;
+            T* top = reinterpret_cast<T*>(p.to) + off;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float of = w.acc[db][4 * g + r] * inv_l;
-                        ov[r] = (T)of;
-                        if (JVP) tov[r] = (T)((w.acct[db][4 * g + r] - r_over_l * w.acc[db][4 * g + r]) * inv_l);
+            for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int d = 32 * db + 8 * g + 4 * hh;   // registers 4g..4g+3 are 4 consecutive d
+                    if (d < DV) {
+                        V4 ov, tov;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const float of = w.acc[db][4 * g + r] * inv_l;
+                            ov[r] = (T)of;
+                            if (JVP) tov[r] = (T)((w.acct[db][4 * g + r] - r_over_l * w.acc[db][4 * g + r]) * inv_l);
+                        }
+                        *reinterpret_cast<V4*>(op + d) = ov;
+                        if (JVP) *reinterpret_cast<V4*>(top + d) = tov;
                     }
-                    *reinterpret_cast<V4*>(op + d) = ov;
-                    if (JVP) *reinterpret_cast<V4*>(top + d) = tov;
                 }
             }
         }
-        if (p.lse && hh == 0) p.lse[(int64_t)bh * p.Lq + row] = (w.m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
     }
 }
 
@@ -660,6 +658,14 @@ int mode_of(const cosmos_attn_desc* d) {
 size_t tile_bytes_of(const cosmos_attn_desc* d) {
     const TileGeom g(d->d_qk, d->d_v, mode_of(d) == MODE_JVP_FULL);
     return (size_t)g.tile_frags * kFragBytes;
+}
+// LDS of the attention kernel: K ring, V ring, P^T/H^T hand-over buffers, rescale factors (AttnCfg::LDS_BYTES)
+size_t lds_bytes_of(const cosmos_attn_desc* d) {
+    const int mode = mode_of(d);
+    const TileGeom g(d->d_qk, d->d_v, mode == MODE_JVP_FULL);
+    const size_t kp = (size_t)g.kpart_frags * kFragBytes, vp = (size_t)(g.tile_frags - g.kpart_frags) * kFragBytes;
+    const size_t ph = (size_t)(mode == MODE_FWD ? 2 : 4) * kFragBytes;
+    return kRingK * kp + kRingV * vp + 2 * 4 * ph + 2 * 4 * 256;
 }
 int n_tiles_of(const cosmos_attn_desc* d) { return (d->Lkv + kBlockN - 1) / kBlockN; }
 // workspace = packed tiles [B*H][n_tiles][tile bytes]
@@ -726,7 +732,7 @@ COSMOS_ATTN_API int cosmos_attn_pack_kv(const cosmos_attn_desc* d, void* workspa
     pp.v_sb = d->v_stride[0]; pp.v_sh = d->v_stride[1]; pp.v_sl = d->v_stride[2];
     pp.out = (uint4*)workspace;
     pp.H = d->H; pp.Lkv = d->Lkv; pp.dqk = d->d_qk; pp.dv = d->d_v; pp.n_tiles = n_tiles_of(d);
-    hipLaunchKernelGGL(pack_kv_kernel, dim3((pp.n_tiles + 1) / 2, d->B * d->H), dim3(kThreads), 0, (hipStream_t)stream, pp);
+    hipLaunchKernelGGL(pack_kv_kernel, dim3((pp.n_tiles + 1) / 2, d->B * d->H), dim3(kPackThreads), 0, (hipStream_t)stream, pp);
     return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
 }
 
@@ -748,13 +754,13 @@ COSMOS_ATTN_API int cosmos_attn_run(const cosmos_attn_desc* d, const void* works
     ap.key_lens = d->key_lens;
     ap.H = d->H; ap.Lq = d->Lq; ap.Lkv = d->Lkv; ap.n_tiles = n_tiles_of(d); ap.causal = d->causal;
     ap.sm_scale = d->sm_scale; ap.scale_log2 = d->sm_scale * 1.4426950408889634f;
-    const size_t lds = 4 * tile_bytes_of(d);   // rings of 4 K parts + 4 V parts
+    const size_t lds = lds_bytes_of(d);
     if (hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
         (void)hipGetLastError();
         return COSMOS_ATTN_LAUNCH_FAILED;
     }
     const int n_qt = (d->Lq + kBlockM - 1) / kBlockM;
-    hipLaunchKernelGGL(fn, dim3(n_qt, d->B * d->H), dim3(kThreads), lds, (hipStream_t)stream, ap);
+    hipLaunchKernelGGL(fn, dim3(n_qt, d->B * d->H), dim3(kAttnThreads), lds, (hipStream_t)stream, ap);
     return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
 }
 
