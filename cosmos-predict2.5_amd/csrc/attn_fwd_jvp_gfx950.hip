@@ -171,7 +171,7 @@ struct AttnCfg {
     static constexpr int TILE_BYTES = KP_BYTES + VP_BYTES;
     static constexpr int DK_OFF = K_FR * kFragBytes;     // inside the K part
     static constexpr int DVT_OFF = VT_FR * kFragBytes;   // inside the V part
-    static constexpr int KP_LOADS = (KP_FR + 7) / 8, VP_LOADS = (VP_FR + 7) / 8;   // per wavefront per tile (8 wavefronts)
+    static constexpr int KP_LOADS = (KP_FR + 3) / 4, VP_LOADS = (VP_FR + 3) / 4;   // per output wavefront per tile (they issue all fills)
     static constexpr int GROUP_LOADS = KP_LOADS + VP_LOADS;
     static constexpr int MFMA_PER_C = FULL ? 3 : (JVP ? 2 : 1);
     // P^T (and H^T) of one tile as MFMA B operands: 2 (4) fragments per score wavefront, double-buffered
@@ -201,13 +201,18 @@ template <int IMM>
 __device__ __forceinline__ void lds_load(__amdgpu_buffer_rsrc_t rsrc, char* dst, int lane_off, int src) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane_off, src, IMM, 0);
 }
+template <int LOADS>
+__device__ __forceinline__ void issue_part(__amdgpu_buffer_rsrc_t rsrc, char* dst, int lane_off, int src) {
+    lds_load<0>(rsrc, dst, lane_off, src);
+    if (LOADS > 1) lds_load<kFragBytes>(rsrc, dst, lane_off, src);
+    if (LOADS > 2) lds_load<2 * kFragBytes>(rsrc, dst, lane_off, src);
+    if (LOADS > 3) lds_load<3 * kFragBytes>(rsrc, dst, lane_off, src);
+}
 template <typename C>
 __device__ __forceinline__ void issue_group(const LoadJob& j) {
-    static_assert(C::KP_LOADS <= 2 && C::VP_LOADS <= 2, "a part has at most 16 fragments");
-    lds_load<0>(j.rsrc, j.v_dst, j.lane_off, j.v_src);
-    if (C::VP_LOADS > 1) lds_load<kFragBytes>(j.rsrc, j.v_dst, j.lane_off, j.v_src);
-    lds_load<0>(j.rsrc, j.k_dst, j.lane_off, j.k_src);
-    if (C::KP_LOADS > 1) lds_load<kFragBytes>(j.rsrc, j.k_dst, j.lane_off, j.k_src);
+    static_assert(C::KP_LOADS <= 4 && C::VP_LOADS <= 4, "a part has at most 16 fragments");
+    issue_part<C::VP_LOADS>(j.rsrc, j.v_dst, j.lane_off, j.v_src);
+    issue_part<C::KP_LOADS>(j.rsrc, j.k_dst, j.lane_off, j.k_src);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -223,8 +228,8 @@ struct ScoreWave {
     static constexpr int PD = COSMOS_ATTN_PREFETCH_GROUPS;   // LDS operand fetches run this many chunks ahead of use
 
     // Scores of one tile as this lane sees them: its query column x 16 of the tile's 32 keys (element e is key
-    // 8 (e/4) + 4 (lane/32) + e%4 of the tile).
-    struct Scores { float s[16]; float ds[16]; };
+    // 8 (e/4) + 4 (lane/32) + e%4 of the tile) -- the accumulator registers of the score MFMAs themselves.
+    struct Scores { f32x16 s, ds; };
 
     V8 qf[NC], tqf[NC];
     float m_run, l_run, r_run;
@@ -235,18 +240,22 @@ struct ScoreWave {
         return *reinterpret_cast<const V8*>(base + frag * kFragBytes + lane * 16);
     }
 
+    __device__ __forceinline__ static float lane_max(const Scores& x) {
+        float mx = x.s[0];
+#pragma unroll
+        for (int e = 1; e < 16; ++e) mx = fmaxf(mx, x.s[e]);
+        return mx;
+    }
+
     // Rare path (last tile of a ragged / padded key range, causal diagonal): masked keys (>= kv_len, or above the
-    // diagonal when causal) get score -inf, hence p = 0 and H = 0.  Returns the lane-local max of the masked scores.
-    __device__ __forceinline__ static float mask_scores(Scores& x, int key0, int kv_len, bool causal, int row) {
-        float mx = -INFINITY;
+    // diagonal when causal) get score -inf, hence p = 0 and H = 0.
+    __device__ __forceinline__ static void mask_scores(Scores& x, int key0, int kv_len, bool causal, int row) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const int key = key0 + 8 * (e >> 2) + (e & 3);
             const bool ok = key < kv_len && (!causal || key <= row);
             x.s[e] = ok ? x.s[e] : -INFINITY;
-            mx = fmaxf(mx, x.s[e]);
         }
-        return mx;
     }
 
     // Fold a tile's lane-local score max into the running max.  Returns the factor by which everything accumulated
@@ -281,38 +290,37 @@ struct ScoreWave {
         }
     }
 
-    // One step: softmax of the tile whose scores are in `x` (already folded into m_run) and, if `next`, the scores
-    // of the next tile from `kpart` into `x`.  P^T / H^T go to `ph_out`, `alpha` to `alpha_out`.
-    // Returns the lane-local max of the new scores.
-    __device__ __forceinline__ float step(Scores& x, const char* kpart, unsigned ph_out, unsigned alpha_out, float alpha) {
+    // One step: softmax of the tile whose scores are in `x` (already folded into m_run; `alpha` is the rescale
+    // factor that goes with it) interleaved with the score MFMAs of the next tile (K part `kpart`) into `xn`.
+    // P^T / H^T go to `ph_out`, `alpha` to `alpha_out` (LDS addresses).
+    __device__ __forceinline__ void step(const Scores& x, Scores& xn, const char* kpart, unsigned ph_out, unsigned alpha_out, float alpha) {
         V8 pf[2], hf[2];
         V8 fa[NC], fb[NC];
         asm volatile("ds_write_b32 %0, %1" ::"v"(alpha_out + 4 * lane), "v"(alpha) : "memory");
 #pragma unroll
         for (int i = 0; i < PD && i < NC; ++i) { fa[i] = lds_frag(kpart, i); if (FULL) fb[i] = lds_frag(kpart + C::DK_OFF, i); }
-        f32x16 sn, dsn;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) { sn[e] = 0.f; dsn[e] = 0.f; }
+        for (int e = 0; e < 16; ++e) { xn.s[e] = 0.f; xn.ds[e] = 0.f; }
         constexpr int EPC = 16 / NC;   // softmax elements dealt out per chunk (NC <= 8)
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             SCHED_FENCE();
             if (c + PD < NC) { fa[c + PD] = lds_frag(kpart, c + PD); if (FULL) fb[c + PD] = lds_frag(kpart + C::DK_OFF, c + PD); }
             SCHED_FENCE();
-            sn = mfma32(fa[c], qf[c], sn);
+            xn.s = mfma32(fa[c], qf[c], xn.s);
 #pragma unroll
             for (int k = 0; k < EPC; ++k)
                 if (k * C::MFMA_PER_C / EPC == 0) softmax_elem(x, pf, hf, c * EPC + k);
             SCHED_FENCE();
             if (JVP) {
-                dsn = mfma32(fa[c], tqf[c], dsn);
+                xn.ds = mfma32(fa[c], tqf[c], xn.ds);
 #pragma unroll
                 for (int k = 0; k < EPC; ++k)
                     if (k * C::MFMA_PER_C / EPC == 1) softmax_elem(x, pf, hf, c * EPC + k);
                 SCHED_FENCE();
             }
             if (FULL) {
-                dsn = mfma32(fb[c], qf[c], dsn);
+                xn.ds = mfma32(fb[c], qf[c], xn.ds);
 #pragma unroll
                 for (int k = 0; k < EPC; ++k)
                     if (k * C::MFMA_PER_C / EPC == 2) softmax_elem(x, pf, hf, c * EPC + k);
@@ -328,36 +336,19 @@ struct ScoreWave {
             asm volatile("ds_write_b128 %0, %1 offset:2048" ::"v"(pa), "v"(hf[0]) : "memory");
             asm volatile("ds_write_b128 %0, %1 offset:3072" ::"v"(pa), "v"(hf[1]) : "memory");
         }
-        float mx = -INFINITY;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            x.s[e] = sn[e];
-            if (JVP) x.ds[e] = dsn[e];
-            mx = fmaxf(mx, x.s[e]);
-        }
-        return mx;
     }
 
-    // scores of the first tile (prologue); returns the lane-local max
-    __device__ __forceinline__ float scores_plain(Scores& x, const char* kpart) const {
-        f32x16 s, ds;
+    // scores of the first tile (prologue)
+    __device__ __forceinline__ void scores_plain(Scores& x, const char* kpart) const {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) { s[e] = 0.f; ds[e] = 0.f; }
+        for (int e = 0; e < 16; ++e) { x.s[e] = 0.f; x.ds[e] = 0.f; }
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const V8 kf = lds_frag(kpart, c);
-            if (JVP) ds = mfma32(kf, tqf[c], ds);
-            s = mfma32(kf, qf[c], s);
-            if (FULL) ds = mfma32(lds_frag(kpart + C::DK_OFF, c), qf[c], ds);
+            if (JVP) x.ds = mfma32(kf, tqf[c], x.ds);
+            x.s = mfma32(kf, qf[c], x.s);
+            if (FULL) x.ds = mfma32(lds_frag(kpart + C::DK_OFF, c), qf[c], x.ds);
         }
-        float mx = -INFINITY;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            x.s[e] = s[e];
-            if (JVP) x.ds[e] = ds[e];
-            mx = fmaxf(mx, x.s[e]);
-        }
-        return mx;
     }
 };
 
@@ -463,7 +454,7 @@ attn_fwd_jvp_kernel(const AttnParams p) {
     const int shift = p.causal ? 0 : (((wg_linear >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
     auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane((u + shift) % n_sweep); };
     auto wrap_inc = [&](int t) { ++t; return t >= n_sweep ? t - n_sweep : t; };
-    const int k_run = ((wave * C::KP_LOADS) % C::KP_FR) * kFragBytes, v_run = ((wave * C::VP_LOADS) % C::VP_FR) * kFragBytes;
+    const int k_run = ((qw * C::KP_LOADS) % C::KP_FR) * kFragBytes, v_run = ((qw * C::VP_LOADS) % C::VP_FR) * kFragBytes;
     // tk / tv: tiles whose K part / V part the group copies; ku / vu: sweep positions that pick the ring slots
     auto make_job = [&](int tk, int ku, int tv, int vu) {
         LoadJob jb;
@@ -475,13 +466,15 @@ attn_fwd_jvp_kernel(const AttnParams p) {
     // Fill stream, in issue order:  K(0) K(1) K(2) [V(0) K(3)] | step 0: [V(1) K(4)] | step 1: [V(2) K(5)] | ...
     // (positions past the end of the sweep wrap around: that data is loaded but never used, so that every
     // wavefront always issues the same number of loads)
+    // The output wavefronts issue all fills (their instruction stream has room; the score wavefronts' has not).
+    if (!score_role) {
 #pragma unroll
-    for (int u = 0; u < 3; ++u) {
-        const LoadJob jb = make_job(tile_at(u), u, 0, 0);
-        lds_load<0>(jb.rsrc, jb.k_dst, jb.lane_off, jb.k_src);
-        if (C::KP_LOADS > 1) lds_load<kFragBytes>(jb.rsrc, jb.k_dst, jb.lane_off, jb.k_src);
+        for (int u = 0; u < 3; ++u) {
+            const LoadJob jb = make_job(tile_at(u), u, 0, 0);
+            issue_part<C::KP_LOADS>(jb.rsrc, jb.k_dst, jb.lane_off, jb.k_src);
+        }
+        issue_group<C>(make_job(tile_at(3), 3, tile_at(0), 0));
     }
-    issue_group<C>(make_job(tile_at(3), 3, tile_at(0), 0));
 
     const bool causal = p.causal != 0;
     // wavefront-uniform: does tile t hold a key some row of this wavefront must not see?
@@ -512,35 +505,36 @@ attn_fwd_jvp_kernel(const AttnParams p) {
         w.l_run = 0.f;         // this lane's partial row sum of p (the two half rows are added in the epilogue)
         w.r_run = 0.f;         // this lane's partial row sum of H
 
-        typename SW::Scores sc;
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): everything issued so far has landed (this wavefront's share)
-        __builtin_amdgcn_s_barrier();
+        typename SW::Scores sc0, sc1;   // scores of the current / next tile, swapping roles every step
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): Q, dQ are here
+        __builtin_amdgcn_s_barrier();         // ... and so is the K part of the first tile
         asm volatile("" ::: "memory");
         float alpha = 1.0f;
-        {
-            float mx = w.scores_plain(sc, kring);
-            const int t0 = tile_at(0);
-            if (need_mask(t0)) mx = SW::mask_scores(sc, t0 * kBlockN + 4 * hh, kv_len, causal, row);
-            if (n_tiles > 0) alpha = w.update_max(mx);
-        }
-        // Step s: softmax of tile s, scores of tile s+1 (K part resident since the barrier at the top of the step).
-        for (int s = 0; s <= n_tiles; ++s) {
-            // own P^T / H^T stores of step s-1 done (lgkmcnt(0)), own fills of V(s-1), K(s+1) landed (vmcnt); the
-            // barrier then says the same of every wavefront, and that every wavefront finished step s-1
-            __builtin_amdgcn_s_waitcnt(WAIT_FILLS & 0xF0FF);
+        // fold a tile's scores into the running max (masking them first where the tile needs it)
+        auto fold = [&](typename SW::Scores& x, int t) {
+            if (need_mask(t)) SW::mask_scores(x, t * kBlockN + 4 * hh, kv_len, causal, row);
+            alpha = w.update_max(SW::lane_max(x));
+        };
+        w.scores_plain(sc0, kring);
+        if (n_tiles > 0) fold(sc0, tile_at(0));
+        // Step s: softmax of tile s (scores in `cur`), scores of tile s+1 into `nxt` (K part resident since the barrier
+        // at the top of the step), statistics of tile s+1.
+        auto body = [&](int s, typename SW::Scores& cur, typename SW::Scores& nxt) {
+            // own P^T / H^T stores of step s-1 done (lgkmcnt(0)); the barrier then says so of every score wavefront,
+            // that the fills of V(s-1), K(s+1) landed, and that every wavefront finished step s-1
+            __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            // V(s+1) overwrites V(s-2), K(s+4) overwrites K(s): both dead since the barrier
-            issue_group<C>(make_job(t_k, s + 4, t_v, s + 1));
             if (s < n_tiles) {
-                float mx = w.step(sc, kring + ((s + 1) % kRingK) * KP_BYTES, lds0 + ph_base + (s & 1) * 4 * C::PH_BYTES,
-                                  lds0 + alpha_base + (s & 1) * 4 * 256, alpha);
-                if (s + 1 < n_tiles) {
-                    if (need_mask(t_v)) mx = SW::mask_scores(sc, t_v * kBlockN + 4 * hh, kv_len, causal, row);
-                    alpha = w.update_max(mx);
-                }
+                w.step(cur, nxt, kring + ((s + 1) % kRingK) * KP_BYTES, lds0 + ph_base + (s & 1) * 4 * C::PH_BYTES,
+                       lds0 + alpha_base + (s & 1) * 4 * 256, alpha);
+                if (s + 1 < n_tiles) fold(nxt, t_v);
             }
-            t_v = wrap_inc(t_v); t_k = wrap_inc(t_k);
+            t_v = wrap_inc(t_v);   // tile at sweep position s + 2
+        };
+        for (int s = 0; s <= n_tiles; s += 2) {
+            body(s, sc0, sc1);
+            if (s + 1 <= n_tiles) body(s + 1, sc1, sc0);
         }
         __builtin_amdgcn_s_waitcnt(0x0070);   // drain the (unused) trailing fills and the last stores
         __builtin_amdgcn_s_barrier();         // the output wavefronts have read the last alpha
