@@ -24,16 +24,17 @@
 //     buffer loads (buffer_load_dwordx4 ... lds, no VGPR staging) and reads fragments back with
 //     conflict-free linear ds_read_b128.  Re-tiling costs one extra read+write of K/V (<1 % of the
 //     call at L=84480) and removes every transpose / swizzle / tail check from the hot loop.
-//   * One workgroup = 4 wavefronts = 128 query rows; 1 wavefront per SIMD with the full 512-register
-//     budget: Q, dQ fragments in VGPRs, both fp32 accumulators pinned to AccVGPRs for the whole sweep.
-//   * The KV sweep is software-pipelined in 32-key steps.  Stage A of a step issues the score MFMAs of
-//     the NEXT tile interleaved with the softmax VALU work of the current one; stage B issues the
-//     P.V-type MFMAs of the current tile interleaved with the rest of the softmax and the AccVGPR ->
-//     VGPR copy-out of the next tile's scores.  LDS holds a ring of four K parts and four V parts
-//     (128 KB at d=128 with tangents); every wavefront issues its quarter of the fills three tiles
-//     ahead, waits with s_waitcnt vmcnt(n) for its own fills of the tile needed next, and one workgroup
-//     barrier per step publishes them.  MFMA operands are prefetched from LDS two MFMA groups ahead,
-//     across step boundaries.
+//   * One workgroup = 128 query rows = 8 wavefronts, two per SIMD, in two ROLES.  A single CDNA wavefront overlaps
+//     its own VALU and MFMA instructions poorly (4 VALU per MFMA already cost 25 % of the MFMA rate), two wavefronts
+//     on one SIMD overlap freely, and one wavefront cannot hold Q, dQ, the scores and both 32 x 128 fp32
+//     accumulators in the 256 registers that two-per-SIMD leaves it.  So wavefront w (< 4) is a SCORE wavefront:
+//     Q, dQ fragments, the score MFMAs of the next tile interleaved with the softmax VALU work of the current one,
+//     the running max / row sums; and wavefront w + 4 (same SIMD) is the OUTPUT wavefront of the same 32 rows: both
+//     accumulators and the P.V-type MFMAs.  P^T, H^T (already 16-bit MFMA B operands) and the rescale factor go
+//     from one to the other through double-buffered LDS slots, one step apart.
+//   * LDS: ring of 4 K parts and ring of 3 V parts (K, dK / V^T, dV^T of 32 keys each), filled 2-3 tiles ahead by
+//     the output wavefronts; hand-over slots; 146 KB at d = 128 with tangents.  One bare s_barrier per 32-key step
+//     publishes fills and hand-over (a __syncthreads() would also drain every wavefront's LDS operand prefetch).
 //   * Query-tile index is the fastest grid dimension, so the 256 workgroups in flight sweep the same
 //     head's K/V images and share them through the per-XCD L2s and the Infinity Cache; workgroups of
 //     one XCD start their (order-free) sweep a few tiles apart so they do not hit one L2 channel at once.
