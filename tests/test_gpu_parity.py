@@ -71,6 +71,19 @@ def test_self_attention_d128(pkg, oracle, gpu, L):
     run_case(pkg, oracle, gpu, (1, 2, L, 128), seed=L)
 
 
+@pytest.mark.parametrize("n_tiles", [1, 2, 3, 4, 5, 7])
+@pytest.mark.parametrize("tangents", ["full", "none"])
+def test_key_tile_counts(pkg, oracle, gpu, n_tiles, tangents):
+    """Whole numbers of 32-key tiles around the LDS ring depths (3 and 4): prologue, wrap-around, drain."""
+    run_case(pkg, oracle, gpu, (1, 2, 96, 128), (1, 2, 32 * n_tiles, 128), seed=n_tiles, tangents=tangents)
+
+
+def test_many_workgroups_rotated_sweeps(pkg, oracle, gpu):
+    """64 workgroups per launch: the sweep of a workgroup starts at tile 2 * ((id / 8) mod 32) and wraps around."""
+    run_case(pkg, oracle, gpu, (2, 4, 1024, 128), (2, 4, 1500, 128), seed=11)
+    run_case(pkg, oracle, gpu, (1, 8, 1024, 64), (1, 8, 700, 64), seed=12, tangents="q")
+
+
 def test_against_torch_sdpa_jvp(pkg, oracle, gpu):
     """The quoted oracle itself (torch math SDPA under torch.func.jvp, fp32) on a mid-size case."""
     q, k, v, tq, tk, tv = oracle.make_inputs((2, 3, 300, 128), seed=5)
