@@ -1,4 +1,4 @@
-"""MI355X-native flash-attention forward + forward-mode JVP for Cosmos-Predict2.5's DiT attention.
+"""MI355X-native flash-attention forward + forward-mode JVP (and backward) for Cosmos-Predict2.5's DiT attention.
 
 The directory name is not a Python identifier; load it with ``__graft_entry__.load_package()``
 (registers it as ``cosmos_predict2_5_amd``).
@@ -8,6 +8,6 @@ from .attention import attention as attention_forward
 from .attn_op import HipAttnOp, hip_attention_op
 from .flash_attention_jvp import attention as attention_jvp
 from .flash_attention_jvp import attention_with_lse
-from .ops import fwd_jvp
+from .ops import bwd, fwd_jvp
 
-__all__ = ["attention_jvp", "attention_with_lse", "attention_forward", "HipAttnOp", "hip_attention_op", "fwd_jvp"]
+__all__ = ["attention_jvp", "attention_with_lse", "attention_forward", "HipAttnOp", "hip_attention_op", "fwd_jvp", "bwd"]

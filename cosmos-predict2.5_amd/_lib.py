@@ -16,7 +16,7 @@ from .build import LIB_PATH as _BUILT_LIB_PATH
 # COSMOS_ATTN_LIB: load another build of the same ABI instead of the in-tree one (deployments, A/B timing)
 LIB_PATH = os.environ.get("COSMOS_ATTN_LIB") or _BUILT_LIB_PATH
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 DTYPE_BF16, DTYPE_FP16 = 0, 1
 
 ST_OK, ST_BAD_ARG, ST_BAD_SHAPE, ST_BAD_STRIDE, ST_UNSUPPORTED, ST_WORKSPACE, ST_LAUNCH = range(7)
@@ -53,6 +53,40 @@ class AttnDesc(ctypes.Structure):
     ]
 
 
+class AttnBwdDesc(ctypes.Structure):
+    """Mirror of ``struct cosmos_attn_bwd_desc``."""
+
+    _fields_ = [
+        ("abi_version", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("B", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("Lq", ctypes.c_int32),
+        ("Lkv", ctypes.c_int32),
+        ("d", ctypes.c_int32),
+        ("causal", ctypes.c_int32),
+        ("sm_scale", ctypes.c_float),
+        ("reserved", ctypes.c_int32),
+        ("q", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("o", ctypes.c_void_p),
+        ("dout", ctypes.c_void_p),
+        ("lse", ctypes.c_void_p),
+        ("dq", ctypes.c_void_p),
+        ("dk", ctypes.c_void_p),
+        ("dv", ctypes.c_void_p),
+        ("q_stride", ctypes.c_int64 * 3),
+        ("k_stride", ctypes.c_int64 * 3),
+        ("v_stride", ctypes.c_int64 * 3),
+        ("o_stride", ctypes.c_int64 * 3),
+        ("dout_stride", ctypes.c_int64 * 3),
+        ("dq_stride", ctypes.c_int64 * 3),
+        ("dk_stride", ctypes.c_int64 * 3),
+        ("dv_stride", ctypes.c_int64 * 3),
+    ]
+
+
 EXPORTS = {
     "cosmos_attn_abi_version": (ctypes.c_int, []),
     "cosmos_attn_status_string": (ctypes.c_char_p, [ctypes.c_int]),
@@ -60,6 +94,8 @@ EXPORTS = {
     "cosmos_attn_fwd_jvp": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "cosmos_attn_pack_kv": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "cosmos_attn_run": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "cosmos_attn_bwd_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(AttnBwdDesc)]),
+    "cosmos_attn_bwd": (ctypes.c_int, [ctypes.POINTER(AttnBwdDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
 }
 
 _lib = None

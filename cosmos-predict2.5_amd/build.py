@@ -14,14 +14,13 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_ROOT = os.path.dirname(PKG_DIR)
 LIB_NAME = "libcosmos_attn_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
-SOURCES = [os.path.join(PKG_DIR, "csrc", "attn_fwd_jvp_gfx950.hip")]
+SOURCES = [os.path.join(PKG_DIR, "csrc", name) for name in ("attn_fwd_jvp_gfx950.hip", "attn_bwd_gfx950.hip")]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     "-fvisibility=hidden",
     # packed fp32 VALU ops are kept off for all device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -35,8 +34,7 @@ def find_hipcc() -> str:
     raise RuntimeError("hipcc not found (set HIPCC or add /opt/rocm/bin to PATH)")
 
 
-def build_library(verbose: bool = True, extra_flags=()) -> str:
-    cmd = [find_hipcc(), *HIPCC_FLAGS, *extra_flags, "-I", os.path.join(REPO_ROOT, "include"), *SOURCES, "-o", LIB_PATH + ".tmp"]
+def _run(cmd, verbose):
     if verbose:
         print("[build]", " ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -45,6 +43,24 @@ def build_library(verbose: bool = True, extra_flags=()) -> str:
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{out}")
     if verbose and out.strip():
         print(out)
+
+
+def build_library(verbose: bool = True, extra_flags=()) -> str:
+    """Compile every source to an object (in parallel), link them into the shared library."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    hipcc = find_hipcc()
+    inc = ["-I", os.path.join(REPO_ROOT, "include")]
+    objs = [src + ".o.tmp" for src in SOURCES]
+    cmds = [[hipcc, *HIPCC_FLAGS, *extra_flags, *inc, "-c", src, "-o", obj] for src, obj in zip(SOURCES, objs)]
+    try:
+        with ThreadPoolExecutor(max_workers=len(cmds)) as pool:
+            list(pool.map(lambda c: _run(c, verbose), cmds))
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH + ".tmp"], verbose)
+    finally:
+        for obj in objs:
+            if os.path.exists(obj):
+                os.remove(obj)
     os.replace(LIB_PATH + ".tmp", LIB_PATH)
     return LIB_PATH
 

@@ -1,0 +1,62 @@
+// Pieces shared by the gfx950 attention kernels (forward + JVP, backward): vector types, the MFMA wrapper, the
+// 1 KB operand-fragment constant, direct-to-LDS loads.  Included inside each translation unit's anonymous namespace.
+#ifndef COSMOS_ATTN_COMMON_GFX950_H
+#define COSMOS_ATTN_COMMON_GFX950_H
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct VecOf;
+template <> struct VecOf<__bf16> { typedef bf16x8 v8; typedef bf16x4 v4; };
+template <> struct VecOf<_Float16> { typedef f16x8 v8; typedef f16x4 v4; };
+
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+constexpr int kFragBytes = 1024;   // one MFMA A-operand fragment: 64 lanes x 16 B
+#ifndef COSMOS_ATTN_PREFETCH_GROUPS
+#define COSMOS_ATTN_PREFETCH_GROUPS 2   // LDS operand fetches run this many MFMA groups ahead of use
+#endif
+#ifndef COSMOS_ATTN_SWEEP_STAGGER
+#define COSMOS_ATTN_SWEEP_STAGGER 2   // tiles between the sweep starts of workgroups that share an L2
+#endif
+
+#define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// What one wavefront copies per step (one "load group"): its share of the V part of one tile and of the K part
+// of another, as VP_LOADS + KP_LOADS wavefront-level direct-to-LDS loads.  buffer_load ... lds (MUBUF) rather than
+// global_load_lds: the compiler's wait-count pass treats the latter as a FLAT access that may touch LDS and then
+// turns every later LDS wait into lgkmcnt(0).  One wavefront-level load moves one fragment: lane l's 16 bytes
+// (voffset = 16 l) land at dst + 16 l.  The share is a contiguous run of fragments (parts with fewer fragments
+// than wavefronts are copied redundantly), so one LDS base (M0) and one scalar offset serve the whole run and the
+// fragment index travels in the instruction's immediate offset, which is added to both addresses.
+struct LoadJob {
+    __amdgpu_buffer_rsrc_t rsrc;
+    int lane_off;            // 16 * lane
+    int k_src, v_src;        // byte offsets of this wavefront's runs in the packed buffer
+    char *k_dst, *v_dst;     // LDS destinations of the runs
+};
+template <int IMM>
+__device__ __forceinline__ void lds_load(__amdgpu_buffer_rsrc_t rsrc, char* dst, int lane_off, int src) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane_off, src, IMM, 0);
+}
+template <int LOADS>
+__device__ __forceinline__ void issue_part(__amdgpu_buffer_rsrc_t rsrc, char* dst, int lane_off, int src) {
+    lds_load<0>(rsrc, dst, lane_off, src);
+    if (LOADS > 1) lds_load<kFragBytes>(rsrc, dst, lane_off, src);
+    if (LOADS > 2) lds_load<2 * kFragBytes>(rsrc, dst, lane_off, src);
+    if (LOADS > 3) lds_load<3 * kFragBytes>(rsrc, dst, lane_off, src);
+}
+
+inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+inline bool strides_ok(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0; }
+inline bool head_dim_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
+
+#endif

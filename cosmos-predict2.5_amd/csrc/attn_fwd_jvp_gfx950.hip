@@ -46,33 +46,11 @@
 
 namespace {
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-
-template <typename T> struct VecOf;
-template <> struct VecOf<__bf16> { typedef bf16x8 v8; typedef bf16x4 v4; };
-template <> struct VecOf<_Float16> { typedef f16x8 v8; typedef f16x4 v4; };
-
-__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
-__device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-}
+#include "attn_common_gfx950.h"
 
 constexpr int kBlockM = 128;       // query rows per workgroup (4 wavefronts x 32)
 constexpr int kBlockN = 32;        // keys per tile
 constexpr int kPackThreads = 256;
-constexpr int kFragBytes = 1024;   // one MFMA A-operand fragment: 64 lanes x 16 B
-#ifndef COSMOS_ATTN_PREFETCH_GROUPS
-#define COSMOS_ATTN_PREFETCH_GROUPS 2
-#endif
-#ifndef COSMOS_ATTN_SWEEP_STAGGER
-#define COSMOS_ATTN_SWEEP_STAGGER 2   // tiles between the sweep starts of workgroups that share an L2
-#endif
 
 enum { MODE_FWD = 0, MODE_JVP_Q = 1, MODE_JVP_FULL = 2 };
 
@@ -154,8 +132,6 @@ struct AttnParams {
 
 extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-#define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
-
 constexpr int kAttnThreads = 512;   // 4 score wavefronts + 4 output wavefronts, two per SIMD
 constexpr int kRingK = 4;           // LDS ring depth, K parts
 constexpr int kRingV = 3;           // LDS ring depth, V parts
@@ -185,30 +161,6 @@ struct AttnCfg {
     static constexpr int LDS_BYTES = ALPHA_OFF + 2 * 4 * 256;
 };
 
-// What one wavefront copies per step (one "load group"): its share of the V part of one tile and of the K part
-// of another, as VP_LOADS + KP_LOADS wavefront-level direct-to-LDS loads.  buffer_load ... lds (MUBUF) rather than
-// global_load_lds: the compiler's wait-count pass treats the latter as a FLAT access that may touch LDS and then
-// turns every later LDS wait into lgkmcnt(0).  One wavefront-level load moves one fragment: lane l's 16 bytes
-// (voffset = 16 l) land at dst + 16 l.  The share is a contiguous run of fragments (parts with fewer fragments
-// than wavefronts are copied redundantly), so one LDS base (M0) and one scalar offset serve the whole run and the
-// fragment index travels in the instruction's immediate offset, which is added to both addresses.
-struct LoadJob {
-    __amdgpu_buffer_rsrc_t rsrc;
-    int lane_off;            // 16 * lane
-    int k_src, v_src;        // byte offsets of this wavefront's runs in the packed buffer
-    char *k_dst, *v_dst;     // LDS destinations of the runs
-};
-template <int IMM>
-__device__ __forceinline__ void lds_load(__amdgpu_buffer_rsrc_t rsrc, char* dst, int lane_off, int src) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane_off, src, IMM, 0);
-}
-template <int LOADS>
-__device__ __forceinline__ void issue_part(__amdgpu_buffer_rsrc_t rsrc, char* dst, int lane_off, int src) {
-    lds_load<0>(rsrc, dst, lane_off, src);
-    if (LOADS > 1) lds_load<kFragBytes>(rsrc, dst, lane_off, src);
-    if (LOADS > 2) lds_load<2 * kFragBytes>(rsrc, dst, lane_off, src);
-    if (LOADS > 3) lds_load<3 * kFragBytes>(rsrc, dst, lane_off, src);
-}
 template <typename C>
 __device__ __forceinline__ void issue_group(const LoadJob& j) {
     static_assert(C::KP_LOADS <= 4 && C::VP_LOADS <= 4, "a part has at most 16 fragments");
@@ -639,9 +591,6 @@ attn_kernel_t pick_dqk(int dqk, int dv, int mode) {
     }
 }
 
-bool head_dim_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
-bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
-bool strides_ok(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0; }
 
 int mode_of(const cosmos_attn_desc* d) {
     if (!d->tq && !d->tk && !d->tv) return MODE_FWD;

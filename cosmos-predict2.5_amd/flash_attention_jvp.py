@@ -45,13 +45,14 @@ class _attention(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *args):
-        # The reference delegates to flash-attn's CUDA backward using the saved (q, k, v, o, lse)
-        # (…jvp_triton.py:505-561).  The gfx950 backward kernel is not built yet; the forward already
-        # saves exactly those tensors (lse = natural-log logsumexp of the scaled scores, [B, H, Lq] fp32).
-        raise NotImplementedError(
-            "backward of the HIP attention is not implemented yet; the saved (q, k, v, o, lse) follow the "
-            "reference's contract"
+        # The reference hands the saved (q, k, v, o, lse) and dout to flash-attn's backward and returns
+        # (dq, dk, dv, None, ...) (…jvp_triton.py:505-561): gradient through o only, equal head dims only.
+        q, k, v, out, softmax_lse = ctx.saved_tensors
+        assert q.shape[-1] == k.shape[-1] and k.shape[-1] == v.shape[-1], (
+            "Backward not supported with different headdim."
         )
+        dq, dk, dv = ops.bwd(q, k, v, out, softmax_lse, dout, causal=ctx.causal, sm_scale=ctx.sm_scale)
+        return dq, dk, dv, None, None, None, None, None
 
 
 attention = _attention.apply

@@ -136,3 +136,68 @@ def fwd_jvp(
     # workspace / converted inputs are freed to torch's caching allocator here; it is stream-ordered on
     # the launch stream, so reuse by later work on this stream is safe.
     return o, to, lse
+
+
+def bwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    o: torch.Tensor,
+    lse: torch.Tensor,
+    dout: torch.Tensor,
+    causal: bool = False,
+    sm_scale: Optional[float] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dq, dk, dv) for the cotangent ``dout`` of o; all tensors ``[B, H, L, d]`` views on one GPU, ``lse`` the
+    forward's ``[B, H, Lq]`` fp32.  Mirrors the reference's ``_attention.backward``
+    (cosmos_predict2/_src/predict2/utils/flash_attention_jvp_triton.py:505-561): equal head dims only (:507-509),
+    outputs allocated like ``torch.empty_like`` of q, k, v (:513).
+    """
+    assert q.shape[-1] == k.shape[-1] and k.shape[-1] == v.shape[-1], "Backward not supported with different headdim."
+    B, H, Lq, d = q.shape
+    Lkv = k.shape[-2]
+    assert k.shape == (B, H, Lkv, d) and v.shape == (B, H, Lkv, d)
+    assert o.shape == q.shape and dout.shape == q.shape and lse.shape == (B, H, Lq)
+    assert d in REFERENCE_HEAD_DIMS
+    if d not in SUPPORTED_HEAD_DIMS:
+        raise NotImplementedError(f"head dim {d}: the HIP kernels are built for {SUPPORTED_HEAD_DIMS}")
+    assert (Lq == Lkv) or (not causal), "Causal cross-attention is currently not supported."
+    if not q.is_cuda:
+        raise RuntimeError("cosmos attention (HIP) needs tensors on a GPU; there is no CPU path")
+    if q.dtype not in _DTYPES:
+        raise NotImplementedError(f"dtype={q.dtype} is not supported (bf16 / fp16)")
+    for x in (k, v, o, dout):
+        assert x.dtype == q.dtype and x.device == q.device
+    ready = lambda x: x if _kernel_ready(x) else x.contiguous()
+    q, k, v, o, dout = (ready(x) for x in (q, k, v, o, dout))
+    lse = lse.to(torch.float32).contiguous()
+    if sm_scale is None:
+        sm_scale = d ** (-0.5)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    if not all(_kernel_ready(x) for x in (dq, dk, dv)):   # empty_like of an exotic view: fall back to plain layouts
+        dq, dk, dv = (torch.empty(x.shape, device=x.device, dtype=x.dtype) for x in (q, k, v))
+
+    desc = _lib.AttnBwdDesc()
+    desc.abi_version = _lib.ABI_VERSION
+    desc.dtype = _DTYPES[q.dtype]
+    desc.B, desc.H, desc.Lq, desc.Lkv, desc.d = B, H, Lq, Lkv, d
+    desc.causal = 1 if causal else 0
+    desc.sm_scale = float(sm_scale)
+    desc.reserved = 0
+    desc.q, desc.k, desc.v, desc.o, desc.dout = (x.data_ptr() for x in (q, k, v, o, dout))
+    desc.lse = lse.data_ptr()
+    desc.dq, desc.dk, desc.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    desc.q_stride, desc.k_stride, desc.v_stride = _strides3(q), _strides3(k), _strides3(v)
+    desc.o_stride, desc.dout_stride = _strides3(o), _strides3(dout)
+    desc.dq_stride, desc.dk_stride, desc.dv_stride = _strides3(dq), _strides3(dk), _strides3(dv)
+
+    lib = _lib.load_library()
+    with torch.cuda.device(q.device):
+        ws_bytes = lib.cosmos_attn_bwd_workspace_bytes(ctypes.byref(desc))
+        if ws_bytes == 0:
+            _lib.raise_for_status(lib.cosmos_attn_bwd(ctypes.byref(desc), None, 0, None) or _lib.ST_BAD_ARG)
+        workspace = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        status = lib.cosmos_attn_bwd(ctypes.byref(desc), workspace.data_ptr(), ws_bytes, stream)
+    _lib.raise_for_status(status)
+    return dq, dk, dv

@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define COSMOS_ATTN_ABI_VERSION 1
+#define COSMOS_ATTN_ABI_VERSION 2
 #define COSMOS_ATTN_API __attribute__((visibility("default")))
 
 /* element types of q,k,v,tangents and of o,to (lse is always fp32) */
@@ -104,6 +104,37 @@ COSMOS_ATTN_API int cosmos_attn_fwd_jvp(const cosmos_attn_desc *desc, void *work
  */
 COSMOS_ATTN_API int cosmos_attn_pack_kv(const cosmos_attn_desc *desc, void *workspace, size_t workspace_bytes, void *stream);
 COSMOS_ATTN_API int cosmos_attn_run(const cosmos_attn_desc *desc, const void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Backward (reverse mode through O only).  Replaces the flash-attn calls of `_attention.backward`
+ * (JVP:505-561: `_flash_attn_backward` JVP:514-531, `_flash_attn_varlen_backward` JVP:538-559): inputs q, k, v, the
+ * forward's o and lse (`ctx.saved_tensors`, JVP:506) and dout; outputs dq, dk, dv (JVP:561).  Equal head dims are
+ * required like the reference (JVP:507-509); causal needs Lq == Lkv (the forward's JVP:446).  Tensors are [B, H, L, d]
+ * addressed through element strides (batch, head, row), innermost stride 1; every tensor has its own strides, so the
+ * transposed views the reference hands to flash-attn (JVP:515-523) need no copies.
+ */
+typedef struct cosmos_attn_bwd_desc {
+    int32_t abi_version;     /* COSMOS_ATTN_ABI_VERSION */
+    int32_t dtype;           /* enum cosmos_attn_dtype: element type of q, k, v, o, dout, dq, dk, dv */
+    int32_t B, H;
+    int32_t Lq, Lkv;
+    int32_t d;               /* head dim of q, k and v, in {16,32,64,128} */
+    int32_t causal;
+    float sm_scale;          /* the forward's softmax scale (`ctx.sm_scale`, JVP:499) */
+    int32_t reserved;        /* 0 */
+
+    const void *q, *k, *v, *o, *dout;   /* device */
+    const float *lse;        /* [B,H,Lq] fp32 contiguous, as written by the forward */
+    void *dq, *dk, *dv;      /* outputs, device */
+    int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3], dout_stride[3];
+    int64_t dq_stride[3], dk_stride[3], dv_stride[3];
+} cosmos_attn_bwd_desc;
+
+/* Bytes of device workspace `cosmos_attn_bwd` needs (per-row statistics and the re-tiled query and key streams). */
+COSMOS_ATTN_API size_t cosmos_attn_bwd_workspace_bytes(const cosmos_attn_bwd_desc *desc);
+
+/* dq, dk, dv from dout.  Asynchronous on `stream`, no atomics (bitwise reproducible); returns a status code. */
+COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc *desc, void *workspace, size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -27,6 +27,11 @@ Functions
                         with its rounding points (P and H rounded to the input
                         half type before the P.V-type products, JVP:134-146).
                         Pinned against ``closed_form``.
+``sdpa_grads_torch``    torch autograd of math-SDPA in fp32: (dq, dk, dv) for a cotangent
+                        of the output -- the oracle of the backward.
+``grads_closed_form``   numpy fp64 closed form of the backward.  Pinned against
+                        ``sdpa_grads_torch``, finite differences of ``closed_form`` and the
+                        adjoint identity <dO, jvp> = <grads, tangents>.
 ``rows_oracle``         fp32 torch closed form on a block of query rows against
                         the full K/V -- rows are independent, so this is exact
                         and is what large-L parity and the CPU baseline use.
@@ -180,6 +185,53 @@ def closed_form(q, k, v, tq=None, tk=None, tv=None, sm_scale=None, causal=False,
     if tv is not None:
         dO = dO + np.einsum("bhqk,bhkd->bhqd", P, tv)
     return O, dO, lse
+
+
+def sdpa_grads_torch(q, k, v, dout, sm_scale=None, causal=False):
+    """(dq, dk, dv) = reverse-mode gradients of math scaled_dot_product_attention w.r.t. q, k, v for the output
+    cotangent ``dout``, fp32 on CPU (torch autograd).  The oracle the backward tolerance is quoted against; what the
+    reference obtains from flash-attn in ``_attention.backward`` (JVP:505-561) and checks against autograd of naive
+    attention in its own procedure (JVP:567-607).
+    """
+    import torch
+    import torch.nn.functional as F
+    from torch.nn.attention import SDPBackend, sdpa_kernel
+
+    q, k, v = (x.detach().to("cpu", torch.float32).requires_grad_(True) for x in (q, k, v))
+    dout = dout.detach().to("cpu", torch.float32)
+    with sdpa_kernel(SDPBackend.MATH):
+        o = F.scaled_dot_product_attention(q, k, v, is_causal=causal, scale=sm_scale)
+    dq, dk, dv = torch.autograd.grad(o, (q, k, v), dout)
+    return dq, dk, dv
+
+
+def grads_closed_form(q, k, v, dout, sm_scale=None, causal=False):
+    """fp64 closed form of the backward.  Returns (dQ, dK, dV) as numpy float64.
+
+        P = softmax(Q K^T s)      dP = dO V^T      D = rowsum(dO * O)      dS = P * (dP - D)
+        dV = P^T dO               dK = s dS^T Q    dQ = s dS K
+
+    (the recurrences flash-attn implements for JVP:514-531; D is the usual rowsum(P * dP) rewritten with O = P V).
+    """
+    q, k, v, dout = (_np64(x) for x in (q, k, v, dout))
+    B, H, Lq, d = q.shape
+    Lkv = k.shape[2]
+    s = (1.0 / math.sqrt(d)) if sm_scale is None else float(sm_scale)
+    S = np.einsum("bhqd,bhkd->bhqk", q, k) * s
+    mask = _valid_mask(B, Lq, Lkv, causal, None)
+    if mask is not None:
+        S = np.where(mask, S, -np.inf)
+    m = S.max(axis=-1, keepdims=True)
+    E = np.exp(S - m)
+    P = E / E.sum(axis=-1, keepdims=True)
+    O = np.einsum("bhqk,bhkd->bhqd", P, v)
+    dP = np.einsum("bhqd,bhkd->bhqk", dout, v)
+    D = (dout * O).sum(axis=-1, keepdims=True)
+    dS = P * (dP - D)
+    dV = np.einsum("bhqk,bhqd->bhkd", P, dout)
+    dK = np.einsum("bhqk,bhqd->bhkd", dS, q) * s
+    dQ = np.einsum("bhqk,bhkd->bhqd", dS, k) * s
+    return dQ, dK, dV
 
 
 # --------------------------------------------------------------------------- #

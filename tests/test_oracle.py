@@ -216,3 +216,47 @@ def test_error_metrics(oracle):
     a = np.array([1.0, 2.0, 2.0])
     ma, rl = oracle.error_metrics(a + np.array([0.0, 0.3, 0.0]), a)
     assert abs(ma - 0.3) < 1e-12 and abs(rl - 0.1) < 1e-12
+
+
+# ------------------------------------------------------------------ backward oracle
+@pytest.mark.parametrize("causal", [False, True])
+def test_grads_closed_form_matches_torch_autograd(oracle, causal):
+    import torch
+
+    q, k, v, tq, _, _ = oracle.make_inputs((1, 2, 37, 16), (1, 2, 37 if causal else 53, 16), seed=5, dtype=torch.float64)
+    dout = tq[..., : v.shape[-1]].clone()   # any cotangent of the output's shape
+    want = oracle.sdpa_grads_torch(q, k, v, dout, sm_scale=0.3, causal=causal)
+    got = oracle.grads_closed_form(q, k, v, dout, sm_scale=0.3, causal=causal)
+    for g, w in zip(got, want):
+        assert np.abs(g - w.double().numpy()).max() < 2e-5   # sdpa_grads_torch computes in fp32
+
+
+def test_grads_closed_form_is_the_adjoint_of_the_jvp(oracle):
+    """<dout, J t> = <J^T dout, t> with the forward-mode closed form (pinned independently) as J."""
+    import torch
+
+    q, k, v, tq, tk, tv = oracle.make_inputs((2, 2, 19, 8), (2, 2, 23, 8), seed=9, dtype=torch.float64)
+    dout = torch.randn(q.shape[:-1] + (v.shape[-1],), generator=torch.Generator().manual_seed(1), dtype=torch.float64)
+    _, jt, _ = oracle.closed_form(q, k, v, tq, tk, tv, sm_scale=0.4)
+    dq, dk, dv = oracle.grads_closed_form(q, k, v, dout, sm_scale=0.4)
+    lhs = float((dout.numpy() * jt).sum())
+    rhs = float((dq * tq.numpy()).sum() + (dk * tk.numpy()).sum() + (dv * tv.numpy()).sum())
+    assert abs(lhs - rhs) <= 1e-10 * max(1.0, abs(lhs))
+
+
+def test_grads_closed_form_matches_finite_differences(oracle):
+    import torch
+
+    q, k, v, _, _, _ = oracle.make_inputs((1, 1, 5, 4), (1, 1, 6, 4), seed=2, dtype=torch.float64)
+    dout = torch.randn(1, 1, 5, 4, generator=torch.Generator().manual_seed(3), dtype=torch.float64)
+    dq, dk, dv = oracle.grads_closed_form(q, k, v, dout, sm_scale=0.5)
+    loss = lambda q_, k_, v_: float((oracle.closed_form(q_, k_, v_, sm_scale=0.5)[0] * dout.numpy()).sum())
+    eps = 1e-6
+    for name, x, g in (("q", q, dq), ("k", k, dk), ("v", v, dv)):
+        for idx in [(0, 0, 0, 0), (0, 0, 2, 3), (0, 0, 4, 1)]:
+            xp, xm = x.clone(), x.clone()
+            xp[idx] += eps; xm[idx] -= eps
+            args_p = {"q": (xp, k, v), "k": (q, xp, v), "v": (q, k, xp)}[name]
+            args_m = {"q": (xm, k, v), "k": (q, xm, v), "v": (q, k, xm)}[name]
+            fd = (loss(*args_p) - loss(*args_m)) / (2 * eps)
+            assert abs(fd - g[idx]) < 1e-6, (name, idx, fd, g[idx])
