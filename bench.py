@@ -1,6 +1,6 @@
 """Benchmark of the attention forward + JVP hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b] [--no-cpu]
 
 A "step" is one call of the hot path (re-tiling kernel + attention kernel, through the Python host and
 the C ABI) over one batch of synthetic tensors that are already resident in HBM.  Default workload: the
@@ -8,7 +8,8 @@ configuration the headline metric is quoted on -- 2B DiT self-attention forward 
 B=1, H=16, L=84480, d=128, bf16.  Prints ONE JSON line.
 
 FLOP accounting is the reference's own (cosmos_predict2/_src/predict2/utils/flash_attention_jvp_triton.py:703-713):
-2*B*H*Lq*Lkv*d per matmul, 2 matmuls forward, 6 forward + JVP.
+2*B*H*Lq*Lkv*d per matmul, 2 matmuls forward, 6 forward + JVP, 5 backward ("2.0 (bwd) + 0.5 (recompute)").
+Workload c3b is the backward pass (dq, dk, dv from dout, with the forward's o and lse) at the c3 shape.
 """
 from __future__ import annotations
 
@@ -39,6 +40,7 @@ WORKLOADS = {
     "c3": ("2B DiT self-attention fwd+JVP bf16 720p B1 H16 L84480 d128", 1, 16, 84480, 84480, 128, "full", False, False),
     "c4": ("14B DiT self-attention fwd+JVP bf16 720p B1 H40 L84480 d128", 1, 40, 84480, 84480, 128, "full", True, False),
     "c5": ("2B DiT text cross-attention fwd+JVP bf16 B2 H16 Lq37440 Lkv512 d128 key-padding tangent-on-q", 2, 16, 37440, 512, 128, "q", False, True),
+    "c3b": ("2B DiT self-attention backward bf16 720p B1 H16 L84480 d128", 1, 16, 84480, 84480, 128, "bwd", False, False),
 }
 
 
@@ -94,6 +96,45 @@ def cpu_baseline(oracle, H, Lkv, d, tangents, rows=512, seed=0):
     }
 
 
+def bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d):
+    """One step = cosmos_attn_bwd (statistics, two stream re-tilings, dK/dV kernel, dQ kernel) through the Python host."""
+    q, k, v, dout, _, _ = make_device_inputs(B, H, Lq, Lkv, d, "q", False, dev)
+    dout = dout * 10.0   # ~N(0, 1)
+    o, _, lse = pkg.fwd_jvp(q, k, v)
+    flops = 5 * 2.0 * B * H * Lq * Lkv * d   # the reference's accounting: 5 matmuls
+    step = lambda: pkg.bwd(q, k, v, o, lse, dout)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / args.steps
+    del out
+    ms = []
+    for i in range(args.steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(); out = step(); e1.record()
+        torch.cuda.synchronize()
+        ms.append(e0.elapsed_time(e1))
+        del out
+    avg = sum(ms) / len(ms)
+    achieved = flops / (avg * 1e-3) / 1e12
+    result = {
+        "metric": "attn backward TFLOP/s & % bf16 MFMA peak @ 2B 720p (L=84480); ms per call",
+        "value": flops / sec / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": desc_txt, "B": B, "H": H, "Lq": Lq, "Lkv": Lkv, "d": d, "flop_per_call": flops,
+                   "executed_matmuls": 7, "pct_of_bf16_mfma_peak": 100.0 * flops / sec / 1e12 / PEAK_BF16_TFLOPS},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "cosmos_attn_bwd (attn_bwd_kernel dK/dV + dQ, 3 small launches)", "kernel_ms_avg": avg, "kernel_ms_min": min(ms)},
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -114,6 +155,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     desc_txt, B, H, Lq, Lkv, d, tangents, rms, padded = WORKLOADS[args.workload]
+    if tangents == "bwd":
+        return bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
     q, k, v, tq, tk, tv = make_device_inputs(B, H, Lq, Lkv, d, tangents, rms, dev)
     key_lens = None
     mean_len = Lkv
