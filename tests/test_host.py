@@ -88,6 +88,61 @@ def test_status_codes_for_bad_descriptors(pkg):
     assert L.status_string(0) == "ok"
 
 
+def good_bwd_desc(pkg, **over):
+    D = pkg._lib.AttnBwdDesc()
+    D.abi_version, D.dtype = pkg._lib.ABI_VERSION, pkg._lib.DTYPE_BF16
+    D.B, D.H, D.Lq, D.Lkv, D.d, D.causal, D.sm_scale, D.reserved = 1, 2, 100, 70, 64, 0, 0.1, 0
+    fake = 0x7F0000000000  # never dereferenced: validation only looks at values
+    for i, name in enumerate(("q", "k", "v", "o", "dout", "lse", "dq", "dk", "dv")):
+        setattr(D, name, fake + 4096 * i)
+    for name, L in (("q", 100), ("k", 70), ("v", 70), ("o", 100), ("dout", 100), ("dq", 100), ("dk", 70), ("dv", 70)):
+        setattr(D, name + "_stride", (ctypes.c_int64 * 3)(2 * L * 64, L * 64, 64))
+    for key, val in over.items():
+        setattr(D, key, val)
+    return D
+
+
+def test_bwd_desc_layout_and_status_codes(pkg):
+    L, lib = pkg._lib, pkg._lib.load_library()
+    # 10 x int32/float, 9 pointers, 8 x 3 int64
+    assert ctypes.sizeof(L.AttnBwdDesc) == 40 + 9 * 8 + 8 * 3 * 8
+    assert L.AttnBwdDesc.q.offset == 40 and L.AttnBwdDesc.dv_stride.offset == 40 + 9 * 8 + 7 * 3 * 8
+    ws = lambda D: lib.cosmos_attn_bwd_workspace_bytes(ctypes.byref(D))
+    run = lambda D: lib.cosmos_attn_bwd(ctypes.byref(D), None, 0, None)
+    D = good_bwd_desc(pkg)
+    # statistics (2 floats per query, rounded up to 1 KB) + query stream (4 tiles of 2*4 + 4*2 + 1 fragments)
+    # + key stream (3 tiles of 2*4 + 2*2 fragments), per (b, h)
+    assert ws(D) == 2048 + 2 * 4 * 17 * 1024 + 2 * 3 * 12 * 1024
+    assert run(D) == L.ST_WORKSPACE
+    cases = [
+        (dict(abi_version=1), L.ST_BAD_ARG),
+        (dict(Lkv=0), L.ST_BAD_ARG),
+        (dict(lse=None), L.ST_BAD_ARG),
+        (dict(dk=None), L.ST_BAD_ARG),
+        (dict(dtype=5), L.ST_UNSUPPORTED),
+        (dict(d=256), L.ST_UNSUPPORTED),
+        (dict(d=48), L.ST_BAD_SHAPE),
+        (dict(causal=1), L.ST_BAD_SHAPE),
+        (dict(dout=0x7F0000000004), L.ST_BAD_STRIDE),
+        (dict(dq_stride=(ctypes.c_int64 * 3)(100 * 66, 100 * 66, 66)), L.ST_BAD_STRIDE),
+    ]
+    for over, want in cases:
+        D = good_bwd_desc(pkg, **over)
+        assert ws(D) == 0, over
+        assert run(D) == want, (over, run(D))
+
+
+def test_backward_argument_checks_mirror_reference(pkg):
+    q = torch.zeros(1, 2, 8, 64, dtype=torch.bfloat16)
+    lse = torch.zeros(1, 2, 8)
+    with pytest.raises(AssertionError, match="different headdim"):   # …jvp_triton.py:507-509
+        pkg.bwd(q, q, q[..., :32], q, lse, q)
+    with pytest.raises(RuntimeError, match="GPU"):                   # no CPU path, no fallback
+        pkg.bwd(q, q, q, q, lse, q)
+    with pytest.raises(AssertionError, match="Causal cross-attention"):
+        pkg.bwd(q, q[:, :, :4], q[:, :, :4], q, lse, q, causal=True)
+
+
 def test_status_to_exception_mapping(pkg):
     L = pkg._lib
     L.raise_for_status(L.ST_OK)
