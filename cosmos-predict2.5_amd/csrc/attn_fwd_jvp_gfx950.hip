@@ -556,13 +556,271 @@ attn_fwd_jvp_kernel(const AttnParams p) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Forward only.  Without tangents a wavefront's whole state (Q fragments, one 32 x d_v accumulator, two score sets)
+// fits the 256 registers that two wavefronts per SIMD leave it, and the softmax VALU work per MFMA is three times
+// that of the tangent modes -- too much for one score wavefront per pair.  So all 8 wavefronts do the same thing,
+// each for its own 32 query rows (256 per workgroup): score MFMAs of the next 32 keys interleaved with the softmax of
+// the current ones, then the P.V MFMAs, with P^T never leaving registers.  The workgroup synchronises (and refills
+// the LDS rings) once per 64 keys: a step is two such half steps.
+constexpr int kSymWaves = 12;        // wavefronts per workgroup, three per SIMD
+constexpr int kSymBlockM = 32 * kSymWaves;     // query rows per workgroup
+constexpr int kSymRing = 4;         // LDS ring depth in steps (pairs of packed tiles), K slots and V slots
+
+template <int DQK, int DV>
+struct SymCfg {
+    static constexpr int NC = DQK / 16, NDB = (DV + 31) / 32;
+    static constexpr int K_FR = NC, VT_FR = 2 * NDB;                       // fragments per packed tile
+    static constexpr int KP_BYTES = K_FR * kFragBytes, VP_BYTES = VT_FR * kFragBytes, TILE_BYTES = KP_BYTES + VP_BYTES;
+    static constexpr int KS_BYTES = 2 * KP_BYTES, VS_BYTES = 2 * VP_BYTES;   // ring slots: the parts of two packed tiles
+    static constexpr int K_LOADS = (2 * K_FR + 7) / 8, V_LOADS = (2 * VT_FR + 7) / 8;   // per wavefront per step
+    static_assert(K_LOADS <= 2 && V_LOADS <= 2 && (K_LOADS == 1 || K_FR % 2 == 0) && (V_LOADS == 1 || VT_FR % 2 == 0), "runs stay inside a tile");
+    static constexpr int GROUP_LOADS = K_LOADS + V_LOADS;
+    static constexpr int KRING_OFF = 0, VRING_OFF = kSymRing * KS_BYTES;
+    static constexpr int LDS_BYTES = VRING_OFF + kSymRing * VS_BYTES;
+};
+
+template <typename T, int DQK, int DV>
+struct SymWave {
+    typedef SymCfg<DQK, DV> C;
+    typedef typename VecOf<T>::v8 V8;
+    static constexpr int NC = C::NC, NDB = C::NDB;
+    static constexpr int NB = 2 * NDB;      // P.V MFMA groups of a tile, (c, db) at index c * NDB + db
+    static constexpr int PD = COSMOS_ATTN_PREFETCH_GROUPS;
+
+    V8 qf[NC];
+    f32x16 acc[NDB];
+    float m_run, l_run, scale_log2;
+    int lane;
+
+    __device__ __forceinline__ V8 lds_frag(const char* base, int frag) const {
+        return *reinterpret_cast<const V8*>(base + frag * kFragBytes + lane * 16);
+    }
+    // this lane's scores of a tile: its query column x 16 of the 32 keys (element e is key 8 (e/4) + 4 (lane/32) + e%4)
+    __device__ __forceinline__ static float lane_max(const f32x16& s) {
+        float mx = s[0];
+#pragma unroll
+        for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s[e]);
+        return mx;
+    }
+    __device__ __forceinline__ static void mask_scores(f32x16& s, int key0, int kv_len, bool causal, int row) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int key = key0 + 8 * (e >> 2) + (e & 3);
+            const bool ok = key < kv_len && (!causal || key <= row);
+            s[e] = ok ? s[e] : -INFINITY;
+        }
+    }
+    // fold the lane-local max of a tile's scores into the running max; returns the rescale factor (1 if no row moved)
+    __device__ __forceinline__ float update_max(float mx) {
+        {
+            const unsigned bits = __builtin_bit_cast(unsigned, mx);
+            const auto sw = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+            mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+        }
+        const float m_new = fmaxf(m_run, mx * scale_log2);
+        float alpha = 1.0f;
+        if (__any(m_new > m_run)) {
+            alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= alpha;
+            m_run = m_new;
+        }
+        return alpha;
+    }
+    __device__ __forceinline__ void scores_plain(f32x16& x, const char* kpart) const {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) x[e] = 0.f;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) x = mfma32(lds_frag(kpart, c), qf[c], x);
+    }
+
+    // Half a step (32 keys).  Stage A: scores of the next tile (K part `kpart`) into `xn`, interleaved with the softmax
+    // of the current one (`x`, already folded into m_run) into the 16-bit operands P^T.  Then rescale by `alpha`
+    // (the factor that goes with `x`) if some row's max moved, and stage B: O^T += V^T P^T over the V part `vpart`.
+    __device__ __forceinline__ void half_step(const f32x16& x, f32x16& xn, const char* kpart, const char* vpart, float alpha) {
+        V8 pf[2];
+        constexpr int EPC = 16 / NC;   // softmax elements dealt out per d chunk
+        V8 fa[NC];
+#pragma unroll
+        for (int i = 0; i < PD && i < NC; ++i) fa[i] = lds_frag(kpart, i);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) xn[e] = 0.f;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            SCHED_FENCE();
+            if (c + PD < NC) fa[c + PD] = lds_frag(kpart, c + PD);
+            SCHED_FENCE();
+            xn = mfma32(fa[c], qf[c], xn);
+#pragma unroll
+            for (int k = 0; k < EPC; ++k) {
+                const int e = c * EPC + k;
+                const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(x[e], scale_log2, -m_run));
+                l_run += p;
+                pf[e >> 3][e & 7] = (T)p;
+            }
+        }
+        SCHED_FENCE();
+        V8 fv[NB];
+#pragma unroll
+        for (int i = 0; i < PD && i < NB; ++i) fv[i] = lds_frag(vpart, 2 * (i % NDB) + i / NDB);
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int i = 0; i < NDB; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][e] *= alpha;
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < NB; ++g) {
+            const int c = g / NDB, db = g % NDB;
+            SCHED_FENCE();
+            if (g + PD < NB) fv[g + PD] = lds_frag(vpart, 2 * ((g + PD) % NDB) + (g + PD) / NDB);
+            SCHED_FENCE();
+            acc[db] = mfma32(fv[g], pf[c], acc[db]);
+        }
+        SCHED_FENCE();
+    }
+};
+
+template <typename T, int DQK, int DV>
+__global__ void __attribute__((amdgpu_flat_work_group_size(64 * kSymWaves, 64 * kSymWaves), amdgpu_waves_per_eu(3, 3)))
+attn_fwd_sym_kernel(const AttnParams p) {
+    typedef SymCfg<DQK, DV> C;
+    typedef SymWave<T, DQK, DV> W;
+    typedef typename VecOf<T>::v8 V8;
+    typedef typename VecOf<T>::v4 V4;
+    constexpr int NC = C::NC, NDB = C::NDB;
+    constexpr int TILE_BYTES = C::TILE_BYTES, KS_BYTES = C::KS_BYTES, VS_BYTES = C::VS_BYTES;
+    // K(s), V(s): the K parts / V parts of the two packed tiles at sweep position s ("step tile" g = tiles 2g, 2g+1).
+    // Step s: half step 0 = scores of tile (s,1) | softmax and P.V of tile (s,0); half step 1 = scores of tile (s+1,0) |
+    // softmax and P.V of tile (s,1).  It reads K(s), K(s+1), V(s) and issues the fills of K(s+3), V(s+3) into the slots
+    // of K(s-1), V(s-1), dead since the barrier.  At the top of step s the fills issued up to step s-2 must have
+    // landed; those of step s-1 may be in flight.
+    constexpr int IN_FLIGHT = C::GROUP_LOADS;
+    constexpr int WAIT_FILLS = (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14) | 0x0F70;
+
+    const int qt = blockIdx.x, bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 31, hh = lane >> 5;
+    const int row0 = qt * kSymBlockM + wave * 32;   // first query row of this wavefront
+    const int row = row0 + j;                       // this lane's query row (lanes l and l^32 share it)
+
+    int kv_len = p.Lkv;
+    if (p.key_lens) { const int kl = p.key_lens[b]; kv_len = kl < kv_len ? (kl < 0 ? 0 : kl) : kv_len; }
+    int n_tiles = (kv_len + kBlockN - 1) / kBlockN;
+    if (p.causal) { const int lim = (qt * kSymBlockM + kSymBlockM + kBlockN - 1) / kBlockN; n_tiles = n_tiles < lim ? n_tiles : lim; }
+    const int n_steps = (n_tiles + 1) / 2;   // (a last step tile that sticks out past n_tiles is masked like any tail)
+
+    char* const kring = smem + C::KRING_OFF;
+    char* const vring = smem + C::VRING_OFF;
+    // reads past the end of the buffer (second tile of a last, odd step) return zeros
+    const __amdgpu_buffer_rsrc_t kv_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(p.kv) + (size_t)bh * p.n_tiles * TILE_BYTES, 0, p.n_tiles * TILE_BYTES, 0x00020000);
+    // sweep order (in step tiles): see attn_fwd_jvp_kernel
+    const int n_sweep = n_steps > 0 ? n_steps : 1;
+    const int wg_linear = blockIdx.x + gridDim.x * blockIdx.y;
+    const int shift = p.causal ? 0 : (((wg_linear >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
+    auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane((u + shift) % n_sweep); };
+    auto wrap_inc = [&](int t) { ++t; return t >= n_sweep ? t - n_sweep : t; };
+    // this wavefront's run of fragments inside a K slot / V slot (never crosses a packed tile)
+    const int kf0 = (wave * C::K_LOADS) % (2 * C::K_FR), vf0 = (wave * C::V_LOADS) % (2 * C::VT_FR);
+    const int k_src_run = (kf0 / C::K_FR) * TILE_BYTES + (kf0 % C::K_FR) * kFragBytes;
+    const int v_src_run = (vf0 / C::VT_FR) * TILE_BYTES + C::KP_BYTES + (vf0 % C::VT_FR) * kFragBytes;
+    auto fill = [&](int g, int u) {
+        if (wave >= 8) return;   // eight wavefronts cover a slot
+        issue_part<C::K_LOADS>(kv_rsrc, kring + (u % kSymRing) * KS_BYTES + kf0 * kFragBytes, lane * 16, g * 2 * TILE_BYTES + k_src_run);
+        issue_part<C::V_LOADS>(kv_rsrc, vring + (u % kSymRing) * VS_BYTES + vf0 * kFragBytes, lane * 16, g * 2 * TILE_BYTES + v_src_run);
+    };
+#pragma unroll
+    for (int u = 0; u < 3; ++u) fill(tile_at(u), u);
+
+    W w;
+    w.lane = lane;
+    w.scale_log2 = p.scale_log2;
+    {
+        const int64_t off = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh + (int64_t)row * p.q_sl + 8 * hh;
+        const T* qp = reinterpret_cast<const T*>(p.q) + off;
+        const bool live = row < p.Lq;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            V8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+            w.qf[c] = live ? *reinterpret_cast<const V8*>(qp + 16 * c) : z;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NDB; ++i) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) w.acc[i][e] = 0.f;
+    }
+    w.m_run = -INFINITY;
+    w.l_run = 0.f;
+
+    const bool causal = p.causal != 0;
+    auto need_mask = [&](int t) { return (t * kBlockN + kBlockN > kv_len) || (causal && (t * kBlockN + kBlockN - 1 > row0)); };
+    float alpha = 1.0f;
+    // fold the scores of packed tile pt into the running max (masking them first where the tile needs it)
+    auto fold = [&](f32x16& x, int pt) {
+        if (need_mask(pt)) W::mask_scores(x, pt * kBlockN + 4 * hh, kv_len, causal, row);
+        alpha = w.update_max(W::lane_max(x));
+    };
+    f32x16 sc0, sc1;   // scores of the current / next tile, swapping roles every half step
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): Q and this wavefront's share of the first fills are here
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    w.scores_plain(sc0, kring);
+    if (n_steps > 0) fold(sc0, 2 * tile_at(0));
+    int g_cur = tile_at(0), g_nxt = tile_at(1), g_fill = tile_at(3);
+    for (int s = 0; s < n_steps; ++s) {
+        __builtin_amdgcn_s_waitcnt(WAIT_FILLS);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        fill(g_fill, s + 3);
+        const char* kslot = kring + (s % kSymRing) * KS_BYTES;
+        const char* vslot = vring + (s % kSymRing) * VS_BYTES;
+        {
+            const float a = alpha;
+            w.half_step(sc0, sc1, kslot + C::KP_BYTES, vslot, a);
+            fold(sc1, 2 * g_cur + 1);
+        }
+        {
+            const float a = alpha;
+            w.half_step(sc1, sc0, kring + ((s + 1) % kSymRing) * KS_BYTES, vslot + C::VP_BYTES, a);
+            if (s + 1 < n_steps) fold(sc0, 2 * g_nxt);
+        }
+        g_cur = g_nxt; g_nxt = wrap_inc(g_nxt); g_fill = wrap_inc(g_fill);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // drain the (unused) trailing fills before the LDS is released
+
+    // ---- epilogue: O = acc / l ; LSE = (m + log2 l) ln 2 ----
+    const float l_tot = w.l_run + __shfl_xor(w.l_run, 32);
+    const float inv_l = 1.0f / l_tot;
+    if (row < p.Lq) {
+        T* op = reinterpret_cast<T*>(p.o) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)row * p.o_sl;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = 32 * db + 8 * g + 4 * hh;   // registers 4g..4g+3 are 4 consecutive d
+                if (d < DV) {
+                    V4 ov;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) ov[r] = (T)(w.acc[db][4 * g + r] * inv_l);
+                    *reinterpret_cast<V4*>(op + d) = ov;
+                }
+            }
+        }
+        if (p.lse && hh == 0) p.lse[(int64_t)bh * p.Lq + row] = (w.m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ host
 typedef void (*attn_kernel_t)(const AttnParams);
 
 template <typename T, int DQK, int DV>
 attn_kernel_t pick_mode(int mode) {
     switch (mode) {
-        case MODE_FWD: return attn_fwd_jvp_kernel<T, DQK, DV, MODE_FWD>;
+        case MODE_FWD: return attn_fwd_sym_kernel<T, DQK, DV>;
         case MODE_JVP_Q: return attn_fwd_jvp_kernel<T, DQK, DV, MODE_JVP_Q>;
         default: return attn_fwd_jvp_kernel<T, DQK, DV, MODE_JVP_FULL>;
     }
@@ -608,7 +866,8 @@ size_t lds_bytes_of(const cosmos_attn_desc* d) {
     const int mode = mode_of(d);
     const TileGeom g(d->d_qk, d->d_v, mode == MODE_JVP_FULL);
     const size_t kp = (size_t)g.kpart_frags * kFragBytes, vp = (size_t)(g.tile_frags - g.kpart_frags) * kFragBytes;
-    const size_t ph = (size_t)(mode == MODE_FWD ? 2 : 4) * kFragBytes;
+    if (mode == MODE_FWD) return (size_t)kSymRing * 2 * (kp + vp);   // SymCfg::LDS_BYTES
+    const size_t ph = 4 * kFragBytes;
     return kRingK * kp + kRingV * vp + 2 * 4 * ph + 2 * 4 * 256;
 }
 int n_tiles_of(const cosmos_attn_desc* d) { return (d->Lkv + kBlockN - 1) / kBlockN; }
@@ -703,8 +962,9 @@ COSMOS_ATTN_API int cosmos_attn_run(const cosmos_attn_desc* d, const void* works
         (void)hipGetLastError();
         return COSMOS_ATTN_LAUNCH_FAILED;
     }
-    const int n_qt = (d->Lq + kBlockM - 1) / kBlockM;
-    hipLaunchKernelGGL(fn, dim3(n_qt, d->B * d->H), dim3(kAttnThreads), lds, (hipStream_t)stream, ap);
+    const int block_m = mode == MODE_FWD ? kSymBlockM : kBlockM;
+    const int n_qt = (d->Lq + block_m - 1) / block_m;
+    hipLaunchKernelGGL(fn, dim3(n_qt, d->B * d->H), dim3(mode == MODE_FWD ? 64 * kSymWaves : kAttnThreads), lds, (hipStream_t)stream, ap);
     return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
 }
 

@@ -208,13 +208,14 @@ def test_attn_op_protocol(pkg, oracle, gpu):
     assert torch.equal(out, pkg.hip_attention_op(q.to(gpu), k.to(gpu), v.to(gpu)))
     o2, to2 = op.forward_jvp(q.to(gpu), k.to(gpu), v.to(gpu), tq.to(gpu))
     o_ref, to_ref, _ = oracle.closed_form(tr(q), tr(k), tr(v), tr(tq))
-    assert torch.equal(o2, out)
+    check(oracle, "HipAttnOp.forward_jvp o", o2, np.ascontiguousarray(o_ref.transpose(0, 2, 1, 3)).reshape(B, S, H * D))
     check(oracle, "HipAttnOp.forward_jvp", to2, np.ascontiguousarray(to_ref.transpose(0, 2, 1, 3)).reshape(B, S, H * D))
 
 
 def test_autograd_function_contract(pkg, oracle, gpu):
     """_attention.apply: positional (q,k,v,tq,tk,tv,causal,sm_scale) -> (o, to); `to` carries no gradient; backward
-    of the HIP path is not built and says so."""
+    runs through o only (tests/test_gpu_backward.py checks the gradients; unequal head dims are refused like the
+    reference, …jvp_triton.py:507-509)."""
     q, k, v, tq, tk, tv = (x.to(gpu) for x in oracle.make_inputs((1, 2, 100, 64), seed=3))
     o, to = pkg.attention_jvp(q, k, v, tq, tk, tv, False, 0.25)
     o_ref, to_ref, _ = oracle.closed_form(q.cpu(), k.cpu(), v.cpu(), tq.cpu(), tk.cpu(), tv.cpu(), sm_scale=0.25)
@@ -223,7 +224,11 @@ def test_autograd_function_contract(pkg, oracle, gpu):
     qg = q.clone().requires_grad_()
     o, to = pkg.attention_jvp(qg, k, v, tq, tk, tv)
     assert o.requires_grad and not to.requires_grad
-    with pytest.raises(NotImplementedError):
+    o.sum().backward()
+    assert qg.grad is not None and qg.grad.shape == q.shape and torch.isfinite(qg.grad.float()).all()
+    q2, k2, v2, tq2, tk2, tv2 = (x.to(gpu) for x in oracle.make_inputs((1, 2, 40, 64), (1, 2, 40, 64), seed=3, dv=32))
+    o, _ = pkg.attention_jvp(q2.requires_grad_(), k2, v2, tq2, tk2, tv2)
+    with pytest.raises(AssertionError, match="different headdim"):
         o.sum().backward()
 
 
@@ -312,19 +317,26 @@ def test_config3_shape_2b_720p_fwd_jvp(pkg, oracle, gpu):
     # run-to-run reproducibility (fixed sweep order, no atomics)
     o2, to2, lse2 = pkg.fwd_jvp(dq, dk, dv, dtq, dtk, dtv)
     assert torch.equal(o, o2) and torch.equal(to, to2) and torch.equal(lse, lse2)
-    # dQ = dK = 0  =>  dO = attention(Q, K, dV), bit for bit (same MFMA sequence on the same operands)
+    # dQ = dK = 0  =>  dO = attention(Q, K, dV): the tangent path reduces to the forward kernel (which walks the keys
+    # 64 at a time instead of 32, so the two differ by rounding, not bit for bit)
     _, to_v, _ = pkg.fwd_jvp(dq, dk, dv, torch.zeros_like(dq), torch.zeros_like(dk), dtv)
     o_dv, _, _ = pkg.fwd_jvp(dq, dk, dtv)
-    assert torch.equal(to_v, o_dv)
+    ma, rl = oracle.error_metrics(to_v.float().cpu()[:, :, ::97], o_dv.float().cpu()[:, :, ::97])
+    print(f" dV-only tangent vs forward of dV: max_abs={ma:.3e} rel_l2={rl:.3e}", flush=True)
+    assert ma <= MAX_ABS and rl <= REL_L2
     # linearity: the q, (k, v) parts of the tangent add up
     _, to_q, _ = pkg.fwd_jvp(dq, dk, dv, dtq)
     _, to_kv, _ = pkg.fwd_jvp(dq, dk, dv, torch.zeros_like(dq), dtk, dtv)
     ma, rl = oracle.error_metrics((to_q.float() + to_kv.float()).cpu()[:, :, ::97], to.float().cpu()[:, :, ::97])
     print(f" linearity: max_abs={ma:.3e} rel_l2={rl:.3e}", flush=True)
     assert ma <= MAX_ABS and rl <= 2 * REL_L2      # three bf16 roundings instead of one
-    # forward-only entry returns the same O and LSE
+    # forward-only entry returns the same O and LSE up to rounding (it walks the keys 64 at a time)
     o3, none, lse3 = pkg.fwd_jvp(dq, dk, dv)
-    assert none is None and torch.equal(o3, o) and torch.equal(lse3, lse)
+    assert none is None
+    ma, rl = oracle.error_metrics(o3.float().cpu()[:, :, ::97], o.float().cpu()[:, :, ::97])
+    print(f" forward-only O vs forward+JVP O: max_abs={ma:.3e} rel_l2={rl:.3e}", flush=True)
+    assert ma <= MAX_ABS and rl <= REL_L2
+    assert (lse3 - lse).abs().max().item() <= LSE_ABS
 
 
 def test_config2_shape_480p_forward_ragged(pkg, oracle, gpu):
