@@ -24,6 +24,10 @@
 #include <stdint.h>
 #include <stddef.h>
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 #include "cosmos_attn_hip.h"
 
 namespace {
@@ -622,10 +626,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
         bp.out1 = d->dv; bp.o1_sb = d->dv_stride[0]; bp.o1_sh = d->dv_stride[1]; bp.o1_sl = d->dv_stride[2];
         bp.out2 = d->dk; bp.o2_sb = d->dk_stride[0]; bp.o2_sh = d->dk_stride[1]; bp.o2_sl = d->dk_stride[2];
         bp.stream = q_img; bp.L_stat = d->Lkv; bp.L_stream = d->Lq; bp.n_tiles = g.n_q_tiles;
-        if (hipFuncSetAttribute((const void*)k_dkdv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds_dkdv) != hipSuccess) {
-            (void)hipGetLastError();
-            return COSMOS_ATTN_LAUNCH_FAILED;
-        }
+        if (!allow_lds((const void*)k_dkdv, g.lds_dkdv)) return COSMOS_ATTN_LAUNCH_FAILED;
         hipLaunchKernelGGL(k_dkdv, dim3((d->Lkv + kBlock - 1) / kBlock, BH), dim3(kBwdThreads), g.lds_dkdv, stream, bp);
     }
     {   // dQ: stationary queries, streamed keys
@@ -634,10 +635,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
         bp.out1 = d->dq; bp.o1_sb = d->dq_stride[0]; bp.o1_sh = d->dq_stride[1]; bp.o1_sl = d->dq_stride[2];
         bp.out2 = nullptr; bp.o2_sb = bp.o2_sh = bp.o2_sl = 0;
         bp.stream = k_img; bp.L_stat = d->Lq; bp.L_stream = d->Lkv; bp.n_tiles = g.n_k_tiles;
-        if (hipFuncSetAttribute((const void*)k_dq, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds_dq) != hipSuccess) {
-            (void)hipGetLastError();
-            return COSMOS_ATTN_LAUNCH_FAILED;
-        }
+        if (!allow_lds((const void*)k_dq, g.lds_dq)) return COSMOS_ATTN_LAUNCH_FAILED;
         hipLaunchKernelGGL(k_dq, dim3((d->Lq + kBlock - 1) / kBlock, BH), dim3(kBwdThreads), g.lds_dq, stream, bp);
     }
     return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;

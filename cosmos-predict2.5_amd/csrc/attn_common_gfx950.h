@@ -55,6 +55,24 @@ __device__ __forceinline__ void issue_part(__amdgpu_buffer_rsrc_t rsrc, char* ds
     if (LOADS > 3) lds_load<3 * kFragBytes>(rsrc, dst, lane_off, src);
 }
 
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per (device, kernel).  A kernel's LDS size is a compile-time
+// constant of its instantiation, so the call never needs repeating; keeping it out of the steady state also keeps
+// the entry points usable while a stream is being captured into a graph.  (Needs <mutex>, <set>, <utility>.)
+inline bool allow_lds(const void* fn, size_t bytes) {
+    static std::mutex mu;
+    static std::set<std::pair<int, const void*>> done;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return false; }
+    std::lock_guard<std::mutex> lock(mu);
+    if (done.count(std::make_pair(dev, fn))) return true;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    done.insert(std::make_pair(dev, fn));
+    return true;
+}
+
 inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 inline bool strides_ok(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0; }
 inline bool head_dim_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }

@@ -42,6 +42,10 @@
 #include <stdint.h>
 #include <stddef.h>
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 #include "cosmos_attn_hip.h"
 
 namespace {
@@ -958,10 +962,7 @@ COSMOS_ATTN_API int cosmos_attn_run(const cosmos_attn_desc* d, const void* works
     ap.H = d->H; ap.Lq = d->Lq; ap.Lkv = d->Lkv; ap.n_tiles = n_tiles_of(d); ap.causal = d->causal;
     ap.sm_scale = d->sm_scale; ap.scale_log2 = d->sm_scale * 1.4426950408889634f;
     const size_t lds = lds_bytes_of(d);
-    if (hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
-        (void)hipGetLastError();
-        return COSMOS_ATTN_LAUNCH_FAILED;
-    }
+    if (!allow_lds((const void*)fn, lds)) return COSMOS_ATTN_LAUNCH_FAILED;
     const int block_m = mode == MODE_FWD ? kSymBlockM : kBlockM;
     const int n_qt = (d->Lq + block_m - 1) / block_m;
     hipLaunchKernelGGL(fn, dim3(n_qt, d->B * d->H), dim3(mode == MODE_FWD ? 64 * kSymWaves : kAttnThreads), lds, (hipStream_t)stream, ap);
