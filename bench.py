@@ -32,7 +32,7 @@ PEAK_BF16_TFLOPS = 256 * 4096 * 2.4e9 / 1e12
 # HBM-side bytes per launch of attn_fwd_jvp_kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # file (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB; factors calibrated with the 1 GiB copy of --copy-calib).
 # Summaries: profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt.  None = not profiled.
-MEASURED_TRAFFIC_BYTES = {"c3": (2 * 2.89402e7 + 681195) * 1024}
+MEASURED_TRAFFIC_BYTES = {"c3": (2 * 2.78902e7 + 681220) * 1024}
 
 WORKLOADS = {
     # name: (description, B, H, Lq, Lkv, d, tangents, rms-normed q/k, key-padding)
