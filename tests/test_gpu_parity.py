@@ -84,6 +84,28 @@ def test_many_workgroups_rotated_sweeps(pkg, oracle, gpu):
     run_case(pkg, oracle, gpu, (1, 8, 1024, 64), (1, 8, 700, 64), seed=12, tangents="q")
 
 
+# ------------------------------------------------------------------ forward only (its own kernel: 384-row workgroups)
+@pytest.mark.parametrize("Lq,Lkv", [(1, 1), (50, 37), (383, 65), (385, 64), (129, 1), (5, 300), (800, 96)])
+def test_forward_only_ragged(pkg, oracle, gpu, Lq, Lkv):
+    run_case(pkg, oracle, gpu, (1, 2, Lq, 128), (1, 2, Lkv, 128), seed=Lq + Lkv, tangents="none")
+
+
+@pytest.mark.parametrize("dqk,dv", [(16, 16), (32, 128), (64, 64), (128, 32), (128, 16)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_forward_only_head_dims(pkg, oracle, gpu, dqk, dv, dtype):
+    run_case(pkg, oracle, gpu, (2, 2, 200, dqk), (2, 2, 333, dqk), dv=dv, seed=dqk + dv, dtype=dtype, tangents="none")
+
+
+@pytest.mark.parametrize("L", [1, 33, 128, 200, 515, 1000])
+def test_forward_only_causal(pkg, oracle, gpu, L):
+    run_case(pkg, oracle, gpu, (1, 2, L, 64), causal=True, seed=L, tangents="none")
+
+
+@pytest.mark.parametrize("lens", [[64, 512], [7, 33], [300, 31], [1, 65]])
+def test_forward_only_key_padding(pkg, oracle, gpu, lens):
+    run_case(pkg, oracle, gpu, (2, 2, 450, 128), (2, 2, 512, 128), key_lens=lens, seed=sum(lens), tangents="none")
+
+
 def test_against_torch_sdpa_jvp(pkg, oracle, gpu):
     """The quoted oracle itself (torch math SDPA under torch.func.jvp, fp32) on a mid-size case."""
     q, k, v, tq, tk, tv = oracle.make_inputs((2, 3, 300, 128), seed=5)
