@@ -35,6 +35,9 @@
 //   * LDS: ring of 4 K parts and ring of 3 V parts (K, dK / V^T, dV^T of 32 keys each), filled 2-3 tiles ahead by
 //     the output wavefronts; hand-over slots; 146 KB at d = 128 with tangents.  One bare s_barrier per 32-key step
 //     publishes fills and hand-over (a __syncthreads() would also drain every wavefront's LDS operand prefetch).
+//   * Forward only (no tangents) runs a different, symmetric kernel (attn_fwd_sym_kernel below): there the softmax
+//     VALU work per MFMA is three times higher and a wavefront's state is small, so 12 wavefronts (three per SIMD)
+//     each do everything for their own 32 rows and P^T never leaves registers.
 //   * Query-tile index is the fastest grid dimension, so the 256 workgroups in flight sweep the same
 //     head's K/V images and share them through the per-XCD L2s and the Infinity Cache; workgroups of
 //     one XCD start their (order-free) sweep a few tiles apart so they do not hit one L2 channel at once.
@@ -366,6 +369,7 @@ struct OutputWave {
 template <typename T, int DQK, int DV, int MODE>
 __global__ void __attribute__((amdgpu_flat_work_group_size(kAttnThreads, kAttnThreads), amdgpu_waves_per_eu(2, 2)))
 attn_fwd_jvp_kernel(const AttnParams p) {
+    static_assert(MODE != MODE_FWD, "forward only is attn_fwd_sym_kernel's job");
     typedef AttnCfg<DQK, DV, MODE> C;
     typedef ScoreWave<T, DQK, DV, MODE> SW;
     typedef OutputWave<T, DQK, DV, MODE> OW;
