@@ -96,6 +96,26 @@ def cpu_baseline(oracle, H, Lkv, d, tangents, rows=512, seed=0):
     }
 
 
+def gemm_reference(dev):
+    """TFLOP/s of torch.matmul (hipBLASLt) on square bf16 operands: context for the roofline fraction."""
+    out = {}
+    for n, reps in ((8192, 20), (16384, 5)):
+        a = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+        b = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+        for _ in range(3):
+            c = a @ b
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            c = a @ b
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        out[f"{n}^3"] = {"ms": ms, "tflops": 2.0 * n ** 3 / ms / 1e9}
+        del a, b, c
+    return out
+
+
 def bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d):
     """One step = cosmos_attn_bwd (statistics, two stream re-tilings, dK/dV kernel, dQ kernel) through the Python host."""
     q, k, v, dout, _, _ = make_device_inputs(B, H, Lq, Lkv, d, "q", False, dev)
@@ -142,6 +162,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--gemm-ref", action="store_true",
+                    help="also time the vendor bf16 GEMM (torch.matmul) at 8192^3 and 16384^3: what dense MFMA work sustains on this box")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run one plain 1 GiB device copy (calibrates FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
     args = ap.parse_args()
@@ -249,6 +271,8 @@ def main():
         dst.copy_(src)  # one elementwise copy kernel: reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
+    if args.gemm_ref:
+        result["gemm_ref"] = gemm_reference(dev)
     if not args.no_cpu:
         del ws, o, to
         oracle = entry.load_oracle()
