@@ -1,6 +1,6 @@
 """Benchmark of the attention forward + JVP hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr] [--no-cpu]
 
 A "step" is one call of the hot path (re-tiling kernel + attention kernel, through the Python host and
 the C ABI) over one batch of synthetic tensors that are already resident in HBM.  Default workload: the
@@ -10,6 +10,8 @@ B=1, H=16, L=84480, d=128, bf16.  Prints ONE JSON line.
 FLOP accounting is the reference's own (cosmos_predict2/_src/predict2/utils/flash_attention_jvp_triton.py:703-713):
 2*B*H*Lq*Lkv*d per matmul, 2 matmuls forward, 6 forward + JVP, 5 backward ("2.0 (bwd) + 0.5 (recompute)").
 Workload c3b is the backward pass (dq, dk, dv from dout, with the forward's o and lse) at the c3 shape.
+Workload nr is the fused RMSNorm + rotary (+ tangent) kernel on one [1, 84480, 16, 128] tensor: HBM-bound, reported
+in GB/s of algorithmic bytes (x, tx read once; y, ty written once; the angle table read once).
 """
 from __future__ import annotations
 
@@ -32,7 +34,8 @@ PEAK_BF16_TFLOPS = 256 * 4096 * 2.4e9 / 1e12
 # HBM-side bytes per launch of attn_fwd_jvp_kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # file (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB; factors calibrated with the 1 GiB copy of --copy-calib).
 # Summaries: profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt.  None = not profiled.
-MEASURED_TRAFFIC_BYTES = {"c3": (2 * 2.78902e7 + 681220) * 1024}
+# nr: norm_rope_kernel, profiles/norm_rope_kernel_bf16_d128_workload_nr.txt.
+MEASURED_TRAFFIC_BYTES = {"c3": (2 * 2.78902e7 + 681220) * 1024, "nr": (2 * 359158.94 + 675840.03) * 1024}
 
 WORKLOADS = {
     # name: (description, B, H, Lq, Lkv, d, tangents, rms-normed q/k, key-padding)
@@ -41,7 +44,10 @@ WORKLOADS = {
     "c4": ("14B DiT self-attention fwd+JVP bf16 720p B1 H40 L84480 d128", 1, 40, 84480, 84480, 128, "full", True, False),
     "c5": ("2B DiT text cross-attention fwd+JVP bf16 B2 H16 Lq37440 Lkv512 d128 key-padding tangent-on-q", 2, 16, 37440, 512, 128, "q", False, True),
     "c3b": ("2B DiT self-attention backward bf16 720p B1 H16 L84480 d128", 1, 16, 84480, 84480, 128, "bwd", False, False),
+    # the step before attention: per-head RMSNorm + rotary embedding of q (or k) with its tangent, one tensor per call
+    "nr": ("2B DiT q RMSNorm+RoPE+tangent bf16 720p B1 S84480 H16 d128", 1, 16, 84480, 84480, 128, "norm_rope", False, False),
 }
+PEAK_HBM_GBS = 8000.0
 
 
 def make_device_inputs(B, H, Lq, Lkv, d, tangents, rms, dev, seed=0):
@@ -155,6 +161,72 @@ def bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d):
     print(json.dumps(result), flush=True)
 
 
+def copy_calibration(dev):
+    """One plain elementwise copy kernel that reads 1 GiB and writes 1 GiB: the known-size launch the FETCH_SIZE /
+    WRITE_SIZE counters are scaled by."""
+    src = torch.empty(1 << 30, device=dev, dtype=torch.uint8).fill_(1)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
+def bench_norm_rope(args, pkg, dev, desc_txt, B, H, S, D):
+    """One step = cosmos_norm_rope on x, tx [B, S, H, D] bf16 -> y, ty (heads-first), through the Python host."""
+    nro = entry.load_norm_rope_oracle()
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn((B, S, H, D), generator=g, device=dev).to(torch.bfloat16)
+    tx = (torch.randn((B, S, H, D), generator=g, device=dev) * 0.1).to(torch.bfloat16)
+    w = (1.0 + 0.1 * torch.randn(D, generator=g, device=dev)).float()
+    angles = torch.from_numpy(nro.rope_angles_3d(24, 44, 80, D)).to(dev)   # 24 x 44 x 80 = 84480 tokens
+    assert angles.shape[0] == S
+    nbytes = 4 * x.numel() * 2 + angles.numel() * 4 + D * 4     # x, tx in; y, ty out; angles; weight
+    step = lambda: pkg.norm_rope(x, w, angles, tx, out_layout="bhsd")
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    # one launch per step: HIP events on the launch stream around the timed region give the average launch duration
+    # (events around a single 0.3 ms launch would mostly time the host getting to the launch)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        out = step()
+    e1.record()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / args.steps
+    avg = e0.elapsed_time(e1) / args.steps
+    achieved = nbytes / (avg * 1e-3) / 1e9
+    result = {
+        "metric": "q/k RMSNorm+RoPE+tangent GB/s of algorithmic bytes @ 2B 720p (S=84480, H=16, d=128); ms per call",
+        "value": nbytes / sec / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": desc_txt, "B": B, "S": S, "H": H, "D": D, "bytes_per_call": nbytes},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": achieved / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get("nr"),
+                     "kernel": "norm_rope_kernel<16, tangent, bf16>", "kernel_ms_avg": avg},
+    }
+    if args.copy_calib:
+        copy_calibration(dev)
+    if not args.no_cpu:
+        # the same step in torch fp32 on the host cores (library rms_norm + rotation under forward AD), on a sample
+        rows = 2048
+        xs, txs, ws, as_ = x[:, :rows].float().cpu(), tx[:, :rows].float().cpu(), w.cpu().numpy(), angles[:rows].cpu().numpy()
+        nro.norm_rope_torch(xs, ws, as_, txs)
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < 5.0 and reps < 20:
+            nro.norm_rope_torch(xs, ws, as_, txs)
+            reps += 1
+        csec = (time.perf_counter() - t0) / reps
+        cbytes = 4 * xs.numel() * 2 + as_.size * 4
+        result["cpu_baseline"] = {"value": cbytes / csec / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                                  "sample": f"torch rms_norm + rotate-half under torch.func.jvp fp32, first {rows} positions x {H} heads, "
+                                            f"{reps} reps, {csec:.4f} s per rep; same 16-bit byte accounting as the GPU figure"}
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -179,6 +251,8 @@ def main():
     desc_txt, B, H, Lq, Lkv, d, tangents, rms, padded = WORKLOADS[args.workload]
     if tangents == "bwd":
         return bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
+    if tangents == "norm_rope":
+        return bench_norm_rope(args, pkg, dev, desc_txt, B, H, Lq, d)
     q, k, v, tq, tk, tv = make_device_inputs(B, H, Lq, Lkv, d, tangents, rms, dev)
     key_lens = None
     mean_len = Lkv
@@ -266,11 +340,7 @@ def main():
         result["config"]["algorithmic_flop_per_call"] = flops_alg
         result["config"]["algorithmic_tflops"] = flops_alg / sec / 1e12
     if args.copy_calib:
-        src = torch.empty(1 << 30, device=dev, dtype=torch.uint8).fill_(1)
-        dst = torch.empty_like(src)
-        dst.copy_(src)  # one elementwise copy kernel: reads 1 GiB, writes 1 GiB
-        torch.cuda.synchronize()
-        del src, dst
+        copy_calibration(dev)
     if args.gemm_ref:
         result["gemm_ref"] = gemm_reference(dev)
     if not args.no_cpu:

@@ -8,6 +8,6 @@ from .attention import attention as attention_forward
 from .attn_op import HipAttnOp, hip_attention_op
 from .flash_attention_jvp import attention as attention_jvp
 from .flash_attention_jvp import attention_with_lse
-from .ops import bwd, fwd_jvp
+from .ops import bwd, fwd_jvp, norm_rope
 
-__all__ = ["attention_jvp", "attention_with_lse", "attention_forward", "HipAttnOp", "hip_attention_op", "fwd_jvp", "bwd"]
+__all__ = ["attention_jvp", "attention_with_lse", "attention_forward", "HipAttnOp", "hip_attention_op", "fwd_jvp", "bwd", "norm_rope"]

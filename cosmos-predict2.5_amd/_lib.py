@@ -87,6 +87,29 @@ class AttnBwdDesc(ctypes.Structure):
     ]
 
 
+class NormRopeDesc(ctypes.Structure):
+    """Mirror of ``struct cosmos_norm_rope_desc``."""
+
+    _fields_ = [
+        ("abi_version", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("B", ctypes.c_int32),
+        ("S", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("eps", ctypes.c_float),
+        ("reserved", ctypes.c_int32),
+        ("x", ctypes.c_void_p),
+        ("tx", ctypes.c_void_p),
+        ("weight", ctypes.c_void_p),
+        ("angles", ctypes.c_void_p),
+        ("y", ctypes.c_void_p),
+        ("ty", ctypes.c_void_p),
+        ("x_stride", ctypes.c_int64 * 3),
+        ("y_stride", ctypes.c_int64 * 3),
+    ]
+
+
 EXPORTS = {
     "cosmos_attn_abi_version": (ctypes.c_int, []),
     "cosmos_attn_status_string": (ctypes.c_char_p, [ctypes.c_int]),
@@ -96,6 +119,7 @@ EXPORTS = {
     "cosmos_attn_run": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "cosmos_attn_bwd_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(AttnBwdDesc)]),
     "cosmos_attn_bwd": (ctypes.c_int, [ctypes.POINTER(AttnBwdDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "cosmos_norm_rope": (ctypes.c_int, [ctypes.POINTER(NormRopeDesc), ctypes.c_void_p]),
 }
 
 _lib = None

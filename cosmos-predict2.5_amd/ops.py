@@ -201,3 +201,63 @@ def bwd(
         status = lib.cosmos_attn_bwd(ctypes.byref(desc), workspace.data_ptr(), ws_bytes, stream)
     _lib.raise_for_status(status)
     return dq, dk, dv
+
+
+def norm_rope(
+    x: torch.Tensor,
+    weight: Optional[torch.Tensor] = None,
+    rope_emb: Optional[torch.Tensor] = None,
+    tx: Optional[torch.Tensor] = None,
+    eps: float = 1e-6,
+    out_layout: str = "bshd",
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Per-head RMSNorm followed by the rotary embedding, and the tangent of both for ``tx``: what the DiT does to q and
+    k between the projections and the attention call (cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:405-415).
+
+    ``x`` (and ``tx``): ``[B, S, H, D]`` 16-bit; ``weight``: RMSNorm's ``[D]`` parameter (None = ones);
+    ``rope_emb``: the angles ``[S, 1, 1, D]`` / ``[S, D]`` of minimal_v4_dit.py:648-658 (None = no rotation, as for
+    cross-attention keys).  Returns ``(y, ty)`` with the shape of ``x``; ``out_layout="bhsd"`` makes the memory
+    heads-first (a ``[B, S, H, D]`` view of it is returned), ready for the attention kernels without a transpose.
+    """
+    assert x.dim() == 4, "x must be [B, S, H, D]"
+    B, S, H, D = x.shape
+    assert D in REFERENCE_HEAD_DIMS
+    if D not in SUPPORTED_HEAD_DIMS:
+        raise NotImplementedError(f"head dim {D}: the HIP kernels are built for {SUPPORTED_HEAD_DIMS}")
+    if x.dtype not in _DTYPES:
+        raise NotImplementedError(f"dtype={x.dtype} is not supported (bf16 / fp16)")
+    if tx is not None:
+        assert tx.shape == x.shape and tx.dtype == x.dtype and tx.device == x.device
+    assert weight is None or weight.shape == (D,)
+    assert rope_emb is None or rope_emb.numel() == S * D, "rope_emb must hold one angle per (position, channel)"
+    if not x.is_cuda:
+        raise RuntimeError("cosmos attention (HIP) needs tensors on a GPU; there is no CPU path")
+    x, tx = _prep_pair(x, tx)
+    if weight is not None:
+        weight = weight.to(device=x.device, dtype=torch.float32).contiguous()
+    if rope_emb is not None:
+        rope_emb = rope_emb.to(device=x.device, dtype=torch.float32).reshape(S, D).contiguous()
+    if out_layout == "bshd":
+        y = torch.empty((B, S, H, D), device=x.device, dtype=x.dtype)
+    elif out_layout == "bhsd":
+        y = torch.empty((B, H, S, D), device=x.device, dtype=x.dtype).transpose(1, 2)
+    else:
+        raise ValueError(f"out_layout={out_layout!r}")
+    ty = torch.empty_like(y) if tx is not None else None
+
+    desc = _lib.NormRopeDesc()
+    desc.abi_version = _lib.ABI_VERSION
+    desc.dtype = _DTYPES[x.dtype]
+    desc.B, desc.S, desc.H, desc.D = B, S, H, D
+    desc.eps = float(eps)
+    desc.reserved = 0
+    desc.x, desc.tx = x.data_ptr(), (tx.data_ptr() if tx is not None else None)
+    desc.weight = weight.data_ptr() if weight is not None else None
+    desc.angles = rope_emb.data_ptr() if rope_emb is not None else None
+    desc.y, desc.ty = y.data_ptr(), (ty.data_ptr() if ty is not None else None)
+    desc.x_stride, desc.y_stride = _strides3(x), _strides3(y)
+    lib = _lib.load_library()
+    with torch.cuda.device(x.device):
+        status = lib.cosmos_norm_rope(ctypes.byref(desc), torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.raise_for_status(status)
+    return y, ty

@@ -9,6 +9,7 @@
  * Reference interfaces replaced (paths relative to the reference checkout):
  *   JVP = cosmos_predict2/_src/predict2/utils/flash_attention_jvp_triton.py
  *   ATT = cosmos_predict2/_src/predict2/networks/attention.py
+ *   networks/... = cosmos_predict2/_src/predict2/networks/...
  */
 #ifndef COSMOS_ATTN_HIP_H
 #define COSMOS_ATTN_HIP_H
@@ -135,6 +136,33 @@ COSMOS_ATTN_API size_t cosmos_attn_bwd_workspace_bytes(const cosmos_attn_bwd_des
 
 /* dq, dk, dv from dout.  Asynchronous on `stream`, no atomics (bitwise reproducible); returns a status code. */
 COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc *desc, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Fused per-head RMSNorm + rotary position embedding, with optional forward-mode tangent: the step before the attention
+ * call in `Attention.compute_qkv` (networks/minimal_v4_dit.py:405-415: `q_norm` / `k_norm` = te.pytorch.RMSNorm(head_dim,
+ * eps=1e-6) :350-356, then TE `apply_rotary_pos_emb(..., tensor_format="bshd", fused=True)` for self-attention :409-414,
+ * with the angles [L,1,1,D] of networks/minimal_v4_dit.py:648-658).
+ *     n = x * rsqrt(mean_d(x^2) + eps) * weight        (rounded to `dtype`, as RMSNorm's output tensor is)
+ *     y = n * cos(angles) + rotate_half(n) * sin(angles)               rotate_half(n) = cat(-n[D/2:], n[:D/2])
+ *     ty = d/de y(x + e tx)|_{e=0}
+ * x, tx: [B, S, H, D] addressed through element strides (batch, sequence, head), innermost stride 1; y, ty likewise with
+ * their own strides (so the result can be written heads-first).  One kernel launch; no workspace.
+ */
+typedef struct cosmos_norm_rope_desc {
+    int32_t abi_version;     /* COSMOS_ATTN_ABI_VERSION */
+    int32_t dtype;           /* enum cosmos_attn_dtype: element type of x, tx, y, ty */
+    int32_t B, S, H, D;      /* D in {16,32,64,128} */
+    float eps;               /* 1e-6 in the DiT */
+    int32_t reserved;        /* 0 */
+    const void *x, *tx;      /* device; tx may be NULL (then ty must be NULL) */
+    const float *weight;     /* [D] fp32 (RMSNorm's gamma), device; NULL = ones */
+    const float *angles;     /* [S, D] fp32 contiguous, device; NULL = no rotation (cross-attention keys, :409) */
+    void *y, *ty;            /* outputs, device */
+    int64_t x_stride[3];     /* (batch, sequence, head) element strides of x and tx */
+    int64_t y_stride[3];     /* of y and ty */
+} cosmos_norm_rope_desc;
+
+COSMOS_ATTN_API int cosmos_norm_rope(const cosmos_norm_rope_desc *desc, void *stream);
 
 #ifdef __cplusplus
 }

@@ -20,6 +20,11 @@ def oracle():
 
 
 @pytest.fixture(scope="session")
+def nr_oracle():
+    return entry.load_norm_rope_oracle()
+
+
+@pytest.fixture(scope="session")
 def pkg():
     """The package with its HIP library loaded; fails loudly when the library is not built."""
     return entry.load_package()

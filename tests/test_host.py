@@ -15,12 +15,12 @@ HEADER = os.path.join(entry.REPO_ROOT, "include", "cosmos_attn_hip.h")
 
 def declared_symbols():
     text = open(HEADER).read()
-    return re.findall(r"COSMOS_ATTN_API\s+[\w\s\*]+?\b(cosmos_attn_\w+)\s*\(", text)
+    return re.findall(r"COSMOS_ATTN_API\s+[\w\s\*]+?\b(cosmos_(?:attn|norm)_\w+)\s*\(", text)
 
 
 def test_header_and_binding_agree(pkg):
     syms = declared_symbols()
-    assert len(syms) >= 6
+    assert len(syms) >= 9
     assert sorted(syms) == sorted(pkg._lib.EXPORTS)
 
 
@@ -141,6 +141,53 @@ def test_backward_argument_checks_mirror_reference(pkg):
         pkg.bwd(q, q, q, q, lse, q)
     with pytest.raises(AssertionError, match="Causal cross-attention"):
         pkg.bwd(q, q[:, :, :4], q[:, :, :4], q, lse, q, causal=True)
+
+
+def test_norm_rope_desc_layout_and_status_codes(pkg):
+    L, lib = pkg._lib, pkg._lib.load_library()
+    # 8 x int32/float, 6 pointers, 2 x 3 int64
+    assert ctypes.sizeof(L.NormRopeDesc) == 32 + 6 * 8 + 2 * 3 * 8
+    assert L.NormRopeDesc.x.offset == 32 and L.NormRopeDesc.y_stride.offset == 32 + 6 * 8 + 3 * 8
+
+    def desc(**over):
+        D = L.NormRopeDesc()
+        D.abi_version, D.dtype, D.B, D.S, D.H, D.D, D.eps = L.ABI_VERSION, L.DTYPE_BF16, 1, 4, 2, 64, 1e-6
+        D.x, D.y = 0x7F0000000000, 0x7F0000100000   # never dereferenced: every case below is rejected on the host
+        D.x_stride = D.y_stride = (ctypes.c_int64 * 3)(4 * 2 * 64, 2 * 64, 64)
+        for k, v in over.items():
+            setattr(D, k, v)
+        return D
+
+    cases = [
+        (dict(abi_version=1), L.ST_BAD_ARG),
+        (dict(S=0), L.ST_BAD_ARG),
+        (dict(y=None), L.ST_BAD_ARG),
+        (dict(tx=0x7F0000200000), L.ST_BAD_ARG),          # a tangent in without a tangent out
+        (dict(eps=-1.0), L.ST_BAD_ARG),
+        (dict(dtype=5), L.ST_UNSUPPORTED),
+        (dict(D=256), L.ST_UNSUPPORTED),
+        (dict(D=48), L.ST_BAD_SHAPE),
+        (dict(x=0x7F0000000004), L.ST_BAD_STRIDE),
+        (dict(angles=0x7F0000300008), L.ST_BAD_STRIDE),
+        (dict(y_stride=(ctypes.c_int64 * 3)(4 * 2 * 66, 2 * 66, 66)), L.ST_BAD_STRIDE),
+    ]
+    for over, want in cases:
+        got = lib.cosmos_norm_rope(ctypes.byref(desc(**over)), None)
+        assert got == want, (over, got)
+
+
+def test_norm_rope_argument_checks(pkg):
+    x = torch.zeros(1, 8, 2, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):                   # no CPU path, no fallback
+        pkg.norm_rope(x)
+    with pytest.raises(AssertionError):
+        pkg.norm_rope(x[0])
+    with pytest.raises(AssertionError):
+        pkg.norm_rope(x, weight=torch.ones(32))
+    with pytest.raises(AssertionError, match="one angle per"):
+        pkg.norm_rope(x, rope_emb=torch.zeros(4, 1, 1, 64))
+    with pytest.raises(NotImplementedError):
+        pkg.norm_rope(torch.zeros(1, 8, 2, 256, dtype=torch.bfloat16))
 
 
 def test_status_to_exception_mapping(pkg):
