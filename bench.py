@@ -1,6 +1,6 @@
 """Benchmark of the attention forward + JVP hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|blk] [--no-cpu]
 
 A "step" is one call of the hot path (re-tiling kernel + attention kernel, through the Python host and
 the C ABI) over one batch of synthetic tensors that are already resident in HBM.  Default workload: the
@@ -46,6 +46,9 @@ WORKLOADS = {
     "c3b": ("2B DiT self-attention backward bf16 720p B1 H16 L84480 d128", 1, 16, 84480, 84480, 128, "bwd", False, False),
     # the step before attention: per-head RMSNorm + rotary embedding of q (or k) with its tangent, one tensor per call
     "nr": ("2B DiT q RMSNorm+RoPE+tangent bf16 720p B1 S84480 H16 d128", 1, 16, 84480, 84480, 128, "norm_rope", False, False),
+    # the whole DiT self-attention module with a tangent: 4 projections (library GEMMs on stacked primal + tangent),
+    # RMSNorm + RoPE (+ tangent) of q and k, attention forward + JVP
+    "blk": ("2B DiT self-attention module fwd+JVP bf16 720p B1 L84480 K2048 H16 d128", 1, 16, 84480, 84480, 128, "module", False, False),
 }
 PEAK_HBM_GBS = 8000.0
 
@@ -161,6 +164,51 @@ def bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d):
     print(json.dumps(result), flush=True)
 
 
+def bench_module(args, pkg, dev, desc_txt, B, H, L, D):
+    """One step = Attention.forward_jvp(x, tx, rope_emb) of the 2B DiT's self-attention module (K = H * D)."""
+    nro = entry.load_norm_rope_oracle()
+    K = H * D
+    torch.manual_seed(0)
+    m = pkg.Attention(K, None, n_heads=H, head_dim=D)
+    m.init_weights()
+    m = m.to(device=dev, dtype=torch.bfloat16).eval()
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn((B, L, K), generator=g, device=dev).to(torch.bfloat16)
+    tx = (torch.randn((B, L, K), generator=g, device=dev) * 0.1).to(torch.bfloat16)
+    rope = torch.from_numpy(nro.rope_angles_3d(24, 44, 80, D)).to(dev).reshape(L, 1, 1, D)
+    flops_gemm = 4 * 2 * 2.0 * B * L * K * K              # q, k, v, output projections on primal and tangent
+    flops_attn = 6 * 2.0 * B * H * L * L * D
+    flops = flops_gemm + flops_attn
+    step = lambda: m.forward_jvp(x, tx, rope_emb=rope)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        out = step()
+    e1.record()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / args.steps
+    avg = e0.elapsed_time(e1) / args.steps
+    del out
+    achieved = flops / (avg * 1e-3) / 1e12
+    result = {
+        "metric": "DiT self-attention module fwd+JVP TFLOP/s & % bf16 MFMA peak @ 2B 720p (L=84480); ms per call",
+        "value": flops / sec / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": desc_txt, "B": B, "L": L, "K": K, "H": H, "d": D, "flop_per_call": flops,
+                   "flop_gemm": flops_gemm, "flop_attention": flops_attn,
+                   "pct_of_bf16_mfma_peak": 100.0 * flops / sec / 1e12 / PEAK_BF16_TFLOPS},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "whole module call (attn_fwd_jvp_kernel dominates)", "kernel_ms_avg": avg},
+    }
+    print(json.dumps(result), flush=True)
+
+
 def copy_calibration(dev):
     """One plain elementwise copy kernel that reads 1 GiB and writes 1 GiB: the known-size launch the FETCH_SIZE /
     WRITE_SIZE counters are scaled by."""
@@ -251,6 +299,8 @@ def main():
     desc_txt, B, H, Lq, Lkv, d, tangents, rms, padded = WORKLOADS[args.workload]
     if tangents == "bwd":
         return bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
+    if tangents == "module":
+        return bench_module(args, pkg, dev, desc_txt, B, H, Lq, d)
     if tangents == "norm_rope":
         return bench_norm_rope(args, pkg, dev, desc_txt, B, H, Lq, d)
     q, k, v, tq, tk, tv = make_device_inputs(B, H, Lq, Lkv, d, tangents, rms, dev)

@@ -6,8 +6,9 @@ The directory name is not a Python identifier; load it with ``__graft_entry__.lo
 from . import _lib  # noqa: F401
 from .attention import attention as attention_forward
 from .attn_op import HipAttnOp, hip_attention_op
+from .dit_attention import Attention
 from .flash_attention_jvp import attention as attention_jvp
 from .flash_attention_jvp import attention_with_lse
 from .ops import bwd, fwd_jvp, norm_rope
 
-__all__ = ["attention_jvp", "attention_with_lse", "attention_forward", "HipAttnOp", "hip_attention_op", "fwd_jvp", "bwd", "norm_rope"]
+__all__ = ["attention_jvp", "attention_with_lse", "attention_forward", "HipAttnOp", "hip_attention_op", "fwd_jvp", "bwd", "norm_rope", "Attention"]

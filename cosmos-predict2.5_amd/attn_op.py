@@ -48,7 +48,9 @@ class HipAttnOp(torch.nn.Module):
 
     def forward(self, query, key, value, *args: Any, **kwargs) -> torch.Tensor:
         del args, kwargs  # e.g. video_size, used only by the sparse (neighbourhood) op in the reference
-        results = attention(query, key, value)
+        # 16-bit inputs keep their type (fp16 stays fp16); anything else is cast to bf16 as in the reference's attention()
+        dtype = query.dtype if query.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
+        results = attention(query, key, value, dtype=dtype)
         return results.flatten(-2)
 
     def forward_jvp(self, query, key, value, t_query, t_key=None, t_value=None):

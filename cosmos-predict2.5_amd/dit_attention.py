@@ -1,0 +1,176 @@
+"""The DiT ``Attention`` module with ``backend="hip"``: projections (library GEMMs), fused RMSNorm + RoPE and the
+attention kernels of this package, with a forward that also carries a tangent.
+
+Reference: ``Attention`` in cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:286-440 -- same constructor
+arguments, sub-module and parameter names (``q_proj``, ``k_proj``, ``v_proj``, ``output_proj``, ``q_norm.weight``,
+``k_norm.weight``: a reference checkpoint's state dict for the module loads as is), ``init_weights``,
+``compute_qkv``, ``compute_attention``, ``forward``, ``set_context_parallel_group``.  What the reference selects
+with ``backend`` in :361-375 is fixed to the HIP op here.
+
+``forward_jvp`` has no counterpart in the reference checkout: its JVP attention kernel
+(utils/flash_attention_jvp_triton.py) ships without the caller that pushes a tangent through the surrounding
+layers.  The rule used here is the plain one: linear layers map the tangent with the same weights (primal and tangent
+go through each GEMM stacked along the batch), RMSNorm + RoPE and attention use their fused JVP kernels.
+
+Reverse mode: ``forward`` supports autograd through the projections and the attention kernels only when no gradient
+has to flow through RMSNorm + RoPE, which has no backward kernel; it refuses instead of silently detaching.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+from torch import nn
+
+from . import ops
+from .attn_op import HipAttnOp
+
+
+class HeadRMSNormWeight(nn.Module):
+    """Holds the ``weight`` of a per-head RMSNorm (``te.pytorch.RMSNorm(head_dim, eps=1e-6)``, minimal_v4_dit.py:350-353);
+    the arithmetic happens in the fused kernel."""
+
+    def __init__(self, head_dim: int, eps: float = 1e-6):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(head_dim))
+
+    def reset_parameters(self) -> None:
+        nn.init.ones_(self.weight)
+
+
+class Attention(nn.Module):
+    def __init__(
+        self,
+        query_dim: int,
+        context_dim=None,
+        n_heads=8,
+        head_dim=64,
+        dropout=0.0,
+        qkv_format: str = "bshd",
+        backend: str = "hip",
+        use_wan_fp32_strategy: bool = False,
+    ) -> None:
+        super().__init__()
+        self.is_selfattn = context_dim is None
+        assert backend in ["hip"], f"Invalid backend: {backend}"
+        assert qkv_format == "bshd", "only the bshd format of the DiT is built"
+        if use_wan_fp32_strategy:
+            raise NotImplementedError("use_wan_fp32_strategy (fp32 q, k after the rotation) is not built: the kernels take 16-bit q, k")
+        self.backend = backend
+        context_dim = query_dim if context_dim is None else context_dim
+        inner_dim = head_dim * n_heads
+        self.n_heads = n_heads
+        self.head_dim = head_dim
+        self.qkv_format = qkv_format
+        self.query_dim = query_dim
+        self.context_dim = context_dim
+        self.use_wan_fp32_strategy = use_wan_fp32_strategy
+
+        self.q_proj = nn.Linear(query_dim, inner_dim, bias=False)
+        self.q_norm = HeadRMSNormWeight(head_dim, eps=1e-6)
+        self.k_proj = nn.Linear(context_dim, inner_dim, bias=False)
+        self.k_norm = HeadRMSNormWeight(head_dim, eps=1e-6)
+        self.v_proj = nn.Linear(context_dim, inner_dim, bias=False)
+        self.v_norm = nn.Identity()
+        self.output_proj = nn.Linear(inner_dim, query_dim, bias=False)
+        self.output_dropout = nn.Dropout(dropout) if dropout > 1e-4 else nn.Identity()
+        self.attn_op = HipAttnOp()
+
+        self._query_dim = query_dim
+        self._context_dim = context_dim
+        self._inner_dim = inner_dim
+
+    def init_weights(self) -> None:
+        """Same initialisation as minimal_v4_dit.py:381-393: truncated normal with std 1/sqrt(fan_in), cut at 3 std."""
+        for lin, fan_in in ((self.q_proj, self._query_dim), (self.k_proj, self._context_dim),
+                            (self.v_proj, self._context_dim), (self.output_proj, self._inner_dim)):
+            std = 1.0 / math.sqrt(fan_in)
+            torch.nn.init.trunc_normal_(lin.weight, std=std, a=-3 * std, b=3 * std)
+        for layer in (self.q_norm, self.k_norm, self.v_norm):
+            if hasattr(layer, "reset_parameters"):
+                layer.reset_parameters()
+
+    # ------------------------------------------------------------------ pieces
+    def _heads(self, t: torch.Tensor) -> torch.Tensor:
+        """``b ... (h d) -> b (...) h d`` (minimal_v4_dit.py:400-403), sequence dims flattened for the kernels."""
+        return t.reshape(t.shape[0], -1, self.n_heads, self.head_dim)
+
+    @staticmethod
+    def _stack(x: torch.Tensor, tx: Optional[torch.Tensor]):
+        """Primal and tangent along the batch, so that a linear layer maps both in one GEMM."""
+        return x if tx is None else torch.cat([x, tx], dim=0)
+
+    @staticmethod
+    def _apply_stacked(lin: nn.Linear, xs: torch.Tensor, has_tangent: bool):
+        y = lin(xs)
+        if not has_tangent:
+            return y, None
+        b = y.shape[0] // 2
+        return y[:b], y[b:]
+
+    def _norm_rope(self, t, norm: HeadRMSNormWeight, rope_emb, tt=None):
+        rope = rope_emb if (self.is_selfattn and rope_emb is not None) else None   # only for self-attention (:409)
+        return ops.norm_rope(t, norm.weight, rope, tt, eps=norm.eps, out_layout="bhsd")
+
+    def _refuse_reverse_mode(self, *tensors) -> None:
+        if torch.is_grad_enabled() and (
+            any(t is not None and t.requires_grad for t in tensors)
+            or any(p.requires_grad for p in (self.q_proj.weight, self.k_proj.weight, self.q_norm.weight, self.k_norm.weight))
+        ):
+            raise NotImplementedError(
+                "reverse mode through the fused RMSNorm + RoPE is not built: call under torch.no_grad() "
+                "(the attention kernels themselves have a backward, see flash_attention_jvp.attention)")
+
+    # ------------------------------------------------------------------ the reference's surface
+    def compute_qkv(self, x, context=None, rope_emb=None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """q, k, v as ``[B, S, H, D]`` (q and k in heads-first memory, ready for the kernels)."""
+        self._refuse_reverse_mode(x, context)
+        context = x if context is None else context
+        q = self._heads(self.q_proj(x))
+        k = self._heads(self.k_proj(context))
+        v = self._heads(self.v_norm(self.v_proj(context)))
+        q, _ = self._norm_rope(q, self.q_norm, rope_emb)
+        k, _ = self._norm_rope(k, self.k_norm, rope_emb)
+        return q, k, v
+
+    def compute_attention(self, q, k, v, video_size=None):
+        result = self.attn_op(q, k, v, video_size=video_size)   # [B, S, H*D]
+        return self.output_dropout(self.output_proj(result))
+
+    def forward(self, x, context: Optional[torch.Tensor] = None, rope_emb: Optional[torch.Tensor] = None, video_size=None):
+        """x: ``[B, Mq, K]`` (or ``[B, T, H, W, K]``); context: ``[B, Mk, Kc]`` or None for self-attention; rope_emb: the
+        angles ``[Mq, 1, 1, D]`` (self-attention only).  Returns ``[B, Mq, K]`` in the shape of x."""
+        q, k, v = self.compute_qkv(x, context, rope_emb=rope_emb)
+        out = self.compute_attention(q, k, v, video_size=video_size)
+        return out.reshape(*x.shape[:-1], out.shape[-1])
+
+    def set_context_parallel_group(self, process_group, ranks, stream):
+        self.attn_op.set_context_parallel_group(process_group, ranks, stream)
+
+    # ------------------------------------------------------------------ forward mode
+    @torch.no_grad()
+    def forward_jvp(self, x, tx, context=None, tcontext=None, rope_emb=None):
+        """``(out, tout)``: the module's output and its directional derivative along ``(tx, tcontext)``.
+        ``tcontext=None`` with a context means the context does not move (text conditioning)."""
+        assert tx is not None and tx.shape == x.shape
+        if isinstance(self.output_dropout, nn.Dropout) and self.training:
+            raise NotImplementedError("forward_jvp with active dropout")
+        xs = self._stack(x, tx)
+        q, tq = self._apply_stacked(self.q_proj, xs, True)
+        if context is None:
+            k, tk = self._apply_stacked(self.k_proj, xs, True)
+            v, tv = self._apply_stacked(self.v_proj, xs, True)
+        else:
+            assert tcontext is None or tcontext.shape == context.shape
+            cs = self._stack(context, tcontext)
+            k, tk = self._apply_stacked(self.k_proj, cs, tcontext is not None)
+            v, tv = self._apply_stacked(self.v_proj, cs, tcontext is not None)
+        h = self._heads
+        q, tq = self._norm_rope(h(q), self.q_norm, rope_emb, h(tq))
+        k, tk = self._norm_rope(h(k), self.k_norm, rope_emb, None if tk is None else h(tk))
+        o, to = self.attn_op.forward_jvp(q, k, h(v), tq, tk, None if tv is None else h(tv))
+        out, tout = self._apply_stacked(self.output_proj, self._stack(o, to), True)
+        shape = (*x.shape[:-1], out.shape[-1])
+        return out.reshape(shape), tout.reshape(shape)

@@ -25,6 +25,11 @@ def nr_oracle():
 
 
 @pytest.fixture(scope="session")
+def dit_oracle():
+    return entry.load_dit_attention_oracle()
+
+
+@pytest.fixture(scope="session")
 def pkg():
     """The package with its HIP library loaded; fails loudly when the library is not built."""
     return entry.load_package()

@@ -1,0 +1,105 @@
+"""GPU parity of the DiT Attention module (backend "hip": library GEMMs + the fused RMSNorm/RoPE kernel + the attention
+kernels, all through the C ABI) and of its forward-mode tangent, against the CPU oracle of the module
+(torch fp32 under torch.func.jvp, pinned in tests/test_oracle_dit_attention.py) on the same 16-bit weights and inputs.
+
+Tolerance: the module chains four 16-bit stages (projection, normalised q/k, attention output, output projection), each
+rounding to 2^-9 relative (bf16); outputs are compared with relative-L2 <= 1e-2 and max-abs <= 3e-2 * max(1, max|want|).
+"""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+REL_L2, MAX_ABS = 1e-2, 3e-2
+
+
+def check(oracle, name, got, want):
+    ma, rl = oracle.error_metrics(got.float().cpu(), want)
+    lim = MAX_ABS * max(1.0, float(want.abs().max()))
+    print(f"  {name}: max_abs={ma:.3e} (limit {lim:.3e}) rel_l2={rl:.3e}", flush=True)
+    assert math.isfinite(ma) and ma <= lim, f"{name}: max-abs {ma} > {lim}"
+    assert rl <= REL_L2, f"{name}: rel-L2 {rl} > {REL_L2}"
+
+
+def build(pkg, gpu, K, Kc, H, D, dtype, seed):
+    torch.manual_seed(seed)
+    m = pkg.Attention(K, Kc, n_heads=H, head_dim=D)
+    m.init_weights()
+    with torch.no_grad():
+        m.q_norm.weight.add_(0.2 * torch.randn(D))
+        m.k_norm.weight.add_(0.2 * torch.randn(D))
+    return m.to(device=gpu, dtype=dtype).eval()
+
+
+def run(pkg, oracle, nr_oracle, dit_oracle, gpu, B, Mq, K, H, D, Mk=None, Kc=None, dtype=torch.bfloat16, seed=0,
+        moving_context=False, rope=True):
+    cross = Kc is not None
+    print(f"module case B={B} Mq={Mq} K={K} H={H} D={D} Mk={Mk} Kc={Kc} {dtype} moving_context={moving_context} seed={seed}", flush=True)
+    m = build(pkg, gpu, K, Kc, H, D, dtype, seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    x = torch.randn(B, Mq, K, generator=g).to(dtype)
+    tx = (torch.randn(B, Mq, K, generator=g) * 0.3).to(dtype)
+    context = torch.randn(B, Mk, Kc, generator=g).to(dtype) if cross else None
+    tcontext = (torch.randn(B, Mk, Kc, generator=g) * 0.3).to(dtype) if (cross and moving_context) else None
+    angles = torch.from_numpy(nr_oracle.rope_angles_3d(1, 1, Mq, D)) if rope else None
+    rope_emb = None if angles is None else angles.reshape(Mq, 1, 1, D).to(gpu)
+    d = lambda t: None if t is None else t.to(gpu)
+    with torch.no_grad():
+        out = m(d(x), d(context), rope_emb=rope_emb)
+    out2, tout = m.forward_jvp(d(x), d(tx), d(context), d(tcontext), rope_emb=rope_emb)
+    torch.cuda.synchronize()
+    assert out.shape == x.shape and out.dtype == dtype and tout.shape == x.shape
+    w = {k: v for k, v in m.state_dict().items()}
+    want, twant = dit_oracle.attention_module_torch(w, x, context, None if angles is None else angles.numpy(), H, D, tx, tcontext)
+    check(oracle, "out", out, want)
+    check(oracle, "out (jvp call)", out2, want)
+    check(oracle, "tout", tout, twant)
+
+
+def test_self_attention_small(pkg, oracle, nr_oracle, dit_oracle, gpu):
+    run(pkg, oracle, nr_oracle, dit_oracle, gpu, B=2, Mq=100, K=256, H=4, D=64)
+
+
+@pytest.mark.parametrize("D,H", [(128, 2), (64, 3), (32, 4)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_self_attention_head_dims(pkg, oracle, nr_oracle, dit_oracle, gpu, D, H, dtype):
+    run(pkg, oracle, nr_oracle, dit_oracle, gpu, B=1, Mq=333, K=H * D, H=H, D=D, dtype=dtype, seed=D)
+
+
+def test_self_attention_without_rope(pkg, oracle, nr_oracle, dit_oracle, gpu):
+    run(pkg, oracle, nr_oracle, dit_oracle, gpu, B=1, Mq=77, K=128, H=2, D=64, rope=False, seed=3)
+
+
+@pytest.mark.parametrize("moving_context", [False, True])
+def test_cross_attention(pkg, oracle, nr_oracle, dit_oracle, gpu, moving_context):
+    # text cross-attention of the DiT: context of another width, no rotation, tangent on x only (or on both)
+    run(pkg, oracle, nr_oracle, dit_oracle, gpu, B=2, Mq=200, K=256, H=2, D=128, Mk=48, Kc=96, moving_context=moving_context, seed=5)
+
+
+def test_dit_block_shape_reduced_length(pkg, oracle, nr_oracle, dit_oracle, gpu):
+    """The 2B DiT's self-attention (K = 2048, 16 heads of 128) at a length the CPU oracle finishes in seconds."""
+    run(pkg, oracle, nr_oracle, dit_oracle, gpu, B=1, Mq=1536, K=2048, H=16, D=128, seed=9)
+
+
+def test_video_shaped_input_and_state_dict_round_trip(pkg, oracle, nr_oracle, dit_oracle, gpu):
+    B, T, Hh, W, K, H, D = 1, 2, 4, 6, 128, 2, 64
+    m = build(pkg, gpu, K, None, H, D, torch.bfloat16, 11)
+    m2 = pkg.Attention(K, None, n_heads=H, head_dim=D).to(device=gpu, dtype=torch.bfloat16).eval()
+    m2.load_state_dict(m.state_dict())
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(B, T, Hh, W, K, generator=g).bfloat16().to(gpu)
+    a = torch.from_numpy(nr_oracle.rope_angles_3d(T, Hh, W, D)).to(gpu)
+    with torch.no_grad():
+        o1, o2 = m(x, rope_emb=a.reshape(-1, 1, 1, D)), m2(x, rope_emb=a.reshape(-1, 1, 1, D))
+    assert o1.shape == x.shape and torch.equal(o1, o2)
+    want, _ = dit_oracle.attention_module_torch(m.state_dict(), x.reshape(B, -1, K), None, a.cpu().numpy(), H, D)
+    check(oracle, "out", o1.reshape(B, -1, K), want)
+
+
+def test_reverse_mode_is_refused_not_detached(pkg, gpu):
+    m = build(pkg, gpu, 128, None, 2, 64, torch.bfloat16, 13)
+    x = torch.randn(1, 16, 128, device=gpu, dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError, match="reverse mode"):
+        m(x)

@@ -190,6 +190,29 @@ def test_norm_rope_argument_checks(pkg):
         pkg.norm_rope(torch.zeros(1, 8, 2, 256, dtype=torch.bfloat16))
 
 
+def test_dit_attention_module_mirrors_reference_surface(pkg):
+    """Constructor arguments, sub-module / parameter names (a reference state dict must load) and refusals."""
+    m = pkg.Attention(64, None, n_heads=2, head_dim=16)
+    assert m.is_selfattn and m.backend == "hip"
+    # parameter names of cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:349-359 (te RMSNorm holds `weight`)
+    assert sorted(m.state_dict()) == ["k_norm.weight", "k_proj.weight", "output_proj.weight", "q_norm.weight",
+                                      "q_proj.weight", "v_proj.weight"]
+    assert m.q_proj.weight.shape == (32, 64) and m.output_proj.weight.shape == (64, 32) and m.q_norm.weight.shape == (16,)
+    c = pkg.Attention(64, 48, n_heads=2, head_dim=16)
+    assert not c.is_selfattn and c.k_proj.weight.shape == (32, 48)
+    m.init_weights()
+    assert float(m.q_proj.weight.abs().max()) <= 3 / 8 + 1e-6 and torch.equal(m.q_norm.weight, torch.ones(16))
+    for name in ("compute_qkv", "compute_attention", "forward", "set_context_parallel_group", "init_weights", "forward_jvp"):
+        assert callable(getattr(m, name))
+    with pytest.raises(AssertionError, match="Invalid backend"):
+        pkg.Attention(64, backend="transformer_engine")
+    with pytest.raises(NotImplementedError):
+        pkg.Attention(64, use_wan_fp32_strategy=True)
+    with pytest.raises(RuntimeError, match="GPU"):          # no CPU path
+        with torch.no_grad():
+            m.bfloat16()(torch.zeros(1, 4, 64, dtype=torch.bfloat16))
+
+
 def test_status_to_exception_mapping(pkg):
     L = pkg._lib
     L.raise_for_status(L.ST_OK)
