@@ -1,6 +1,6 @@
 """Benchmark of the attention forward + JVP hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|blk] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk] [--no-cpu]
 
 A "step" is one call of the hot path (re-tiling kernel + attention kernel, through the Python host and
 the C ABI) over one batch of synthetic tensors that are already resident in HBM.  Default workload: the
@@ -46,6 +46,7 @@ WORKLOADS = {
     "c3b": ("2B DiT self-attention backward bf16 720p B1 H16 L84480 d128", 1, 16, 84480, 84480, 128, "bwd", False, False),
     # the step before attention: per-head RMSNorm + rotary embedding of q (or k) with its tangent, one tensor per call
     "nr": ("2B DiT q RMSNorm+RoPE+tangent bf16 720p B1 S84480 H16 d128", 1, 16, 84480, 84480, 128, "norm_rope", False, False),
+    "nrb": ("2B DiT q RMSNorm+RoPE backward bf16 720p B1 S84480 H16 d128", 1, 16, 84480, 84480, 128, "norm_rope_bwd", False, False),
     # the whole DiT self-attention module with a tangent: 4 projections (library GEMMs on stacked primal + tangent),
     # RMSNorm + RoPE (+ tangent) of q and k, attention forward + JVP
     "blk": ("2B DiT self-attention module fwd+JVP bf16 720p B1 L84480 K2048 H16 d128", 1, 16, 84480, 84480, 128, "module", False, False),
@@ -219,8 +220,9 @@ def copy_calibration(dev):
     del src, dst
 
 
-def bench_norm_rope(args, pkg, dev, desc_txt, B, H, S, D):
-    """One step = cosmos_norm_rope on x, tx [B, S, H, D] bf16 -> y, ty (heads-first), through the Python host."""
+def bench_norm_rope(args, pkg, dev, desc_txt, B, H, S, D, backward=False):
+    """One step = cosmos_norm_rope on x, tx [B, S, H, D] bf16 -> y, ty (heads-first), through the Python host; with
+    ``backward`` one step = cosmos_norm_rope_bwd on x, dy -> dx, dweight (x, dy read once, dx written once)."""
     nro = entry.load_norm_rope_oracle()
     g = torch.Generator(device=dev).manual_seed(0)
     x = torch.randn((B, S, H, D), generator=g, device=dev).to(torch.bfloat16)
@@ -230,6 +232,10 @@ def bench_norm_rope(args, pkg, dev, desc_txt, B, H, S, D):
     assert angles.shape[0] == S
     nbytes = 4 * x.numel() * 2 + angles.numel() * 4 + D * 4     # x, tx in; y, ty out; angles; weight
     step = lambda: pkg.norm_rope(x, w, angles, tx, out_layout="bhsd")
+    if backward:
+        dy = tx.transpose(1, 2).contiguous().transpose(1, 2)       # the gradient arrives in heads-first memory
+        nbytes = 3 * x.numel() * 2 + angles.numel() * 4 + D * 4   # x, dy in; dx out; angles; weight (partial sums: 2.7 MB)
+        step = lambda: pkg.norm_rope_bwd(x, w, angles, dy)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -246,18 +252,20 @@ def bench_norm_rope(args, pkg, dev, desc_txt, B, H, S, D):
     avg = e0.elapsed_time(e1) / args.steps
     achieved = nbytes / (avg * 1e-3) / 1e9
     result = {
-        "metric": "q/k RMSNorm+RoPE+tangent GB/s of algorithmic bytes @ 2B 720p (S=84480, H=16, d=128); ms per call",
+        "metric": ("q/k RMSNorm+RoPE backward" if backward else "q/k RMSNorm+RoPE+tangent") +
+                  " GB/s of algorithmic bytes @ 2B 720p (S=84480, H=16, d=128); ms per call",
         "value": nbytes / sec / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": desc_txt, "B": B, "S": S, "H": H, "D": D, "bytes_per_call": nbytes},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": achieved / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get("nr"),
-                     "kernel": "norm_rope_kernel<16, tangent, bf16>", "kernel_ms_avg": avg},
+                     "frac": achieved / PEAK_HBM_GBS, "traffic": None if backward else MEASURED_TRAFFIC_BYTES.get("nr"),
+                     "kernel": "norm_rope_bwd_kernel<16, bf16> + norm_rope_dweight_kernel" if backward else "norm_rope_kernel<16, tangent, bf16>",
+                     "kernel_ms_avg": avg},
     }
     if args.copy_calib:
         copy_calibration(dev)
-    if not args.no_cpu:
+    if not args.no_cpu and not backward:
         # the same step in torch fp32 on the host cores (library rms_norm + rotation under forward AD), on a sample
         rows = 2048
         xs, txs, ws, as_ = x[:, :rows].float().cpu(), tx[:, :rows].float().cpu(), w.cpu().numpy(), angles[:rows].cpu().numpy()
@@ -301,8 +309,8 @@ def main():
         return bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
     if tangents == "module":
         return bench_module(args, pkg, dev, desc_txt, B, H, Lq, d)
-    if tangents == "norm_rope":
-        return bench_norm_rope(args, pkg, dev, desc_txt, B, H, Lq, d)
+    if tangents in ("norm_rope", "norm_rope_bwd"):
+        return bench_norm_rope(args, pkg, dev, desc_txt, B, H, Lq, d, backward=tangents == "norm_rope_bwd")
     q, k, v, tq, tk, tv = make_device_inputs(B, H, Lq, Lkv, d, tangents, rms, dev)
     key_lens = None
     mean_len = Lkv

@@ -9,6 +9,6 @@ from .attn_op import HipAttnOp, hip_attention_op
 from .dit_attention import Attention
 from .flash_attention_jvp import attention as attention_jvp
 from .flash_attention_jvp import attention_with_lse
-from .ops import bwd, fwd_jvp, norm_rope
+from .ops import bwd, fwd_jvp, norm_rope, norm_rope_bwd
 
-__all__ = ["attention_jvp", "attention_with_lse", "attention_forward", "HipAttnOp", "hip_attention_op", "fwd_jvp", "bwd", "norm_rope", "Attention"]
+__all__ = ["attention_jvp", "attention_with_lse", "attention_forward", "HipAttnOp", "hip_attention_op", "fwd_jvp", "bwd", "norm_rope", "norm_rope_bwd", "Attention"]

@@ -110,6 +110,30 @@ class NormRopeDesc(ctypes.Structure):
     ]
 
 
+class NormRopeBwdDesc(ctypes.Structure):
+    """Mirror of ``struct cosmos_norm_rope_bwd_desc``."""
+
+    _fields_ = [
+        ("abi_version", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("B", ctypes.c_int32),
+        ("S", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("eps", ctypes.c_float),
+        ("reserved", ctypes.c_int32),
+        ("x", ctypes.c_void_p),
+        ("dy", ctypes.c_void_p),
+        ("weight", ctypes.c_void_p),
+        ("angles", ctypes.c_void_p),
+        ("dx", ctypes.c_void_p),
+        ("dweight", ctypes.c_void_p),
+        ("x_stride", ctypes.c_int64 * 3),
+        ("dy_stride", ctypes.c_int64 * 3),
+        ("dx_stride", ctypes.c_int64 * 3),
+    ]
+
+
 EXPORTS = {
     "cosmos_attn_abi_version": (ctypes.c_int, []),
     "cosmos_attn_status_string": (ctypes.c_char_p, [ctypes.c_int]),
@@ -120,6 +144,8 @@ EXPORTS = {
     "cosmos_attn_bwd_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(AttnBwdDesc)]),
     "cosmos_attn_bwd": (ctypes.c_int, [ctypes.POINTER(AttnBwdDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "cosmos_norm_rope": (ctypes.c_int, [ctypes.POINTER(NormRopeDesc), ctypes.c_void_p]),
+    "cosmos_norm_rope_bwd_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(NormRopeBwdDesc)]),
+    "cosmos_norm_rope_bwd": (ctypes.c_int, [ctypes.POINTER(NormRopeBwdDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
 }
 
 _lib = None

@@ -16,6 +16,26 @@ import torch
 from . import ops
 
 
+class _AttentionFn(torch.autograd.Function):
+    """Forward-only attention on ``[B, S, H, D]`` tensors with a reverse-mode rule: the forward keeps o and the
+    log-sum-exp, the backward is the HIP backward (equal head dims only)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, causal, softmax_scale):
+        o, _, lse = ops.fwd_jvp(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
+                                causal=causal, sm_scale=softmax_scale, out_layout="blhd", need_lse=True)
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.causal, ctx.softmax_scale = causal, softmax_scale
+        return o.transpose(1, 2)
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, o, lse = ctx.saved_tensors
+        t = lambda x: x.transpose(1, 2)
+        dq, dk, dv = ops.bwd(t(q), t(k), t(v), o, lse, t(dout), causal=ctx.causal, sm_scale=ctx.softmax_scale)
+        return t(dq), t(dk), t(dv), None, None
+
+
 def attention(
     q,
     k,
@@ -41,6 +61,9 @@ def attention(
     v = v.to(dtype)
     if q_scale is not None:
         q = q * q_scale
+
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        return _AttentionFn.apply(q, k, v, causal, softmax_scale)   # the SDPA path of the reference is differentiable too
 
     # [B, S, H, D] -> heads-first views (no copy); the kernel writes [B, S, H, D] memory directly
     o, _, _ = ops.fwd_jvp(

@@ -220,6 +220,174 @@ norm_rope_kernel_t pick(int d) {
     }
 }
 
+// ------------------------------------------------------------------------------------------------ reverse mode
+// Given dy = dL/dy:   dn = R^T dy (the rotation by the negated angles; the 16-bit rounding of n is passed straight through)
+//                     dx = r (g dn) - x r^3 mean_d(x g dn),      dweight[j] = sum over rows of dn[j] x[j] r.
+// Same thread layout as the forward kernel.  dweight: every thread sums its heads, the block's thread groups are added
+// in a fixed order through LDS, and each block writes one row of partial sums; norm_rope_dweight_kernel adds the rows
+// (fixed order again: the result is bitwise reproducible, no atomics).
+struct NormRopeBwdParams {
+    const uint16_t *x, *dy;
+    uint16_t* dx;
+    const float* weight;         // [D] or null (ones)
+    const float* angles;         // [S, D] or null (no rotation)
+    float* partials;             // [blocks, D] or null (no dweight wanted)
+    int64_t x_sb, x_ss, x_sh, g_sb, g_ss, g_sh, o_sb, o_ss, o_sh;   // strides of x, dy, dx
+    int B, S, H, D;
+    float eps;
+    int heads_per_unit, head_groups;
+    int64_t units;
+};
+
+template <int TPR, bool BF16>
+__global__ void __launch_bounds__(kThreads) norm_rope_bwd_kernel(const NormRopeBwdParams p) {
+    constexpr int D = TPR * 8;
+    constexpr int HS = kHeadsPerStep;
+    constexpr int UPB = kThreads / TPR;          // units (thread groups) per block
+    __shared__ float red[UPB * D];               // 8 KB for every D
+    const int ug = threadIdx.x / TPR;
+    const int64_t unit = (int64_t)blockIdx.x * UPB + ug;
+    const int part = threadIdx.x % TPR;
+    const bool live = unit < p.units;
+    const int64_t uu = live ? unit : 0;
+    const int h0 = (int)(uu % p.head_groups) * p.heads_per_unit;
+    const int s = (int)((uu / p.head_groups) % p.S);
+    const int b = (int)(uu / ((int64_t)p.head_groups * p.S));
+    const int n_heads = live ? min(p.heads_per_unit, p.H - h0) : 0;
+    const uint16_t* xp = p.x + (int64_t)b * p.x_sb + (int64_t)s * p.x_ss + (int64_t)h0 * p.x_sh + 4 * part;
+    const uint16_t* gp = p.dy + (int64_t)b * p.g_sb + (int64_t)s * p.g_ss + (int64_t)h0 * p.g_sh + 4 * part;
+    uint16_t* op = p.dx + (int64_t)b * p.o_sb + (int64_t)s * p.o_ss + (int64_t)h0 * p.o_sh + 4 * part;
+
+    float g[8], sn[8], cs[8], wacc[8];   // [0, 4): the lower-half elements, [4, 8): their partners in the upper half
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        g[i] = p.weight ? p.weight[4 * part + i] : 1.0f;
+        g[4 + i] = p.weight ? p.weight[D / 2 + 4 * part + i] : 1.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) wacc[i] = 0.f;
+    if (p.angles) {
+        const float4 a0 = *reinterpret_cast<const float4*>(p.angles + (int64_t)s * D + 4 * part);
+        const float4 a1 = *reinterpret_cast<const float4*>(p.angles + (int64_t)s * D + D / 2 + 4 * part);
+        const float lo[4] = {a0.x, a0.y, a0.z, a0.w}, hi[4] = {a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sincosf(lo[i], &sn[i], &cs[i]);
+        if (lo[0] == hi[0] && lo[1] == hi[1] && lo[2] == hi[2] && lo[3] == hi[3]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { sn[4 + i] = sn[i]; cs[4 + i] = cs[i]; }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sincosf(hi[i], &sn[4 + i], &cs[4 + i]);
+        }
+    }
+
+    for (int hb = 0; hb < p.heads_per_unit; hb += HS) {
+        uint2 xlo[HS], xhi[HS], glo[HS], ghi[HS];
+#pragma unroll
+        for (int i = 0; i < HS; ++i) {
+            const int hsel = hb + i < n_heads ? hb + i : 0;   // surplus slots re-read the first head, store nothing
+            xlo[i] = *reinterpret_cast<const uint2*>(xp + hsel * p.x_sh);
+            xhi[i] = *reinterpret_cast<const uint2*>(xp + hsel * p.x_sh + D / 2);
+            glo[i] = *reinterpret_cast<const uint2*>(gp + hsel * p.g_sh);
+            ghi[i] = *reinterpret_cast<const uint2*>(gp + hsel * p.g_sh + D / 2);
+        }
+#pragma unroll
+        for (int hh = 0; hh < HS; ++hh) {
+            float x[8], dy[8], dn[8];
+            unpack4<BF16>(xlo[hh], x);
+            unpack4<BF16>(xhi[hh], x + 4);
+            unpack4<BF16>(glo[hh], dy);
+            unpack4<BF16>(ghi[hh], dy + 4);
+            if (p.angles) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    // transpose of  y_lo = n_lo c_lo - n_hi s_lo,  y_hi = n_hi c_hi + n_lo s_hi
+                    dn[i] = dy[i] * cs[i] + dy[4 + i] * sn[4 + i];
+                    dn[4 + i] = dy[4 + i] * cs[4 + i] - dy[i] * sn[i];
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) dn[i] = dy[i];
+            }
+            float ss = 0.f, sg = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { ss += x[i] * x[i]; sg += x[i] * (g[i] * dn[i]); }
+            ss = group_sum<TPR>(ss);
+            sg = group_sum<TPR>(sg);
+            const float r = rsqrtf(ss * (1.0f / D) + p.eps);
+            const float c3 = r * r * r * sg * (1.0f / D);
+            float dx[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dx[i] = g[i] * dn[i] * r - x[i] * c3;
+            if (hb + hh < n_heads) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) wacc[i] += dn[i] * x[i] * r;
+                uint16_t* o = op + (int64_t)(hb + hh) * p.o_sh;
+                *reinterpret_cast<uint2*>(o) = pack4<BF16>(dx);
+                *reinterpret_cast<uint2*>(o + D / 2) = pack4<BF16>(dx + 4);
+            }
+        }
+    }
+    if (p.partials) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            red[ug * D + 4 * part + i] = wacc[i];
+            red[ug * D + D / 2 + 4 * part + i] = wacc[4 + i];
+        }
+        __syncthreads();
+        if (threadIdx.x < D) {
+            float t = 0.f;
+            for (int u = 0; u < UPB; ++u) t += red[u * D + threadIdx.x];
+            p.partials[(int64_t)blockIdx.x * D + threadIdx.x] = t;
+        }
+    }
+}
+
+// dweight[j] = sum over `rows` of partials[row][j]: one block per channel, fixed order within a thread and across threads
+__global__ void __launch_bounds__(kThreads) norm_rope_dweight_kernel(const float* partials, float* dweight, int64_t rows, int D) {
+    __shared__ float red[kThreads];
+    const int j = blockIdx.x;
+    float t = 0.f;
+    for (int64_t r = threadIdx.x; r < rows; r += kThreads) t += partials[r * D + j];
+    red[threadIdx.x] = t;
+    __syncthreads();
+    for (int w = kThreads / 2; w > 0; w >>= 1) {
+        if (threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) dweight[j] = red[0];
+}
+
+typedef void (*norm_rope_bwd_kernel_t)(const NormRopeBwdParams);
+
+template <bool BF16>
+norm_rope_bwd_kernel_t pick_bwd(int d) {
+    switch (d) {
+        case 16: return norm_rope_bwd_kernel<2, BF16>;
+        case 32: return norm_rope_bwd_kernel<4, BF16>;
+        case 64: return norm_rope_bwd_kernel<8, BF16>;
+        case 128: return norm_rope_bwd_kernel<16, BF16>;
+        default: return nullptr;
+    }
+}
+
+// How the rows are dealt out to thread groups: as many heads per group as there are (up to 16) while that leaves enough
+// groups to fill the chip.
+struct UnitPlan { int heads_per_unit, head_groups; int64_t units, blocks; };
+UnitPlan plan_units(int B, int S, int H, int D) {
+    UnitPlan u;
+    const int units_per_block = kThreads / (D / 8);
+    const int64_t enough_units = (int64_t)units_per_block * 4096;
+    u.heads_per_unit = kHeadsPerStep;
+    while (u.heads_per_unit < kMaxHeadsPerUnit && u.heads_per_unit < H &&
+           (int64_t)B * S * ((H + 2 * u.heads_per_unit - 1) / (2 * u.heads_per_unit)) >= enough_units)
+        u.heads_per_unit *= 2;
+    u.head_groups = (H + u.heads_per_unit - 1) / u.heads_per_unit;
+    u.units = (int64_t)B * S * u.head_groups;
+    u.blocks = (u.units + units_per_block - 1) / units_per_block;
+    return u;
+}
+
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 bool strides_ok(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0; }
 
@@ -245,22 +413,63 @@ COSMOS_ATTN_API int cosmos_norm_rope(const cosmos_norm_rope_desc* d, void* strea
     p.y_sb = d->y_stride[0]; p.y_ss = d->y_stride[1]; p.y_sh = d->y_stride[2];
     p.B = d->B; p.S = d->S; p.H = d->H; p.D = d->D;
     p.eps = d->eps;
-    // as many heads per unit as there are (up to 16) while that leaves enough thread groups to fill the chip
-    const int64_t enough_units = (int64_t)(kThreads / (d->D / 8)) * 4096;
-    p.heads_per_unit = kHeadsPerStep;
-    while (p.heads_per_unit < kMaxHeadsPerUnit && p.heads_per_unit < d->H &&
-           (int64_t)d->B * d->S * ((d->H + 2 * p.heads_per_unit - 1) / (2 * p.heads_per_unit)) >= enough_units)
-        p.heads_per_unit *= 2;
-    p.head_groups = (d->H + p.heads_per_unit - 1) / p.heads_per_unit;
-    p.units = (int64_t)d->B * d->S * p.head_groups;
-    const int units_per_block = kThreads / (d->D / 8);
-    const int64_t blocks = (p.units + units_per_block - 1) / units_per_block;
+    const UnitPlan u = plan_units(d->B, d->S, d->H, d->D);
+    p.heads_per_unit = u.heads_per_unit; p.head_groups = u.head_groups; p.units = u.units;
+    const int64_t blocks = u.blocks;
     if (blocks > 0x7FFFFFFF) return COSMOS_ATTN_BAD_SHAPE;
     const bool bf16 = d->dtype == COSMOS_ATTN_BF16;
     norm_rope_kernel_t fn = d->tx ? (bf16 ? pick<true, true>(d->D) : pick<true, false>(d->D))
                                   : (bf16 ? pick<false, true>(d->D) : pick<false, false>(d->D));
     hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
+}
+
+static int validate_norm_rope_bwd(const cosmos_norm_rope_bwd_desc* d) {
+    if (!d || d->abi_version != COSMOS_ATTN_ABI_VERSION) return COSMOS_ATTN_BAD_ARG;
+    if (d->B <= 0 || d->S <= 0 || d->H <= 0) return COSMOS_ATTN_BAD_ARG;
+    if (!d->x || !d->dy || !d->dx) return COSMOS_ATTN_BAD_ARG;
+    if (!(d->eps >= 0.f)) return COSMOS_ATTN_BAD_ARG;
+    if (d->dtype != COSMOS_ATTN_BF16 && d->dtype != COSMOS_ATTN_FP16) return COSMOS_ATTN_UNSUPPORTED;
+    if (d->D == 256) return COSMOS_ATTN_UNSUPPORTED;
+    if (d->D != 16 && d->D != 32 && d->D != 64 && d->D != 128) return COSMOS_ATTN_BAD_SHAPE;
+    if (!aligned16(d->x) || !aligned16(d->dy) || !aligned16(d->dx)) return COSMOS_ATTN_BAD_STRIDE;
+    if (d->angles && !aligned16(d->angles)) return COSMOS_ATTN_BAD_STRIDE;
+    if (!strides_ok(d->x_stride) || !strides_ok(d->dy_stride) || !strides_ok(d->dx_stride)) return COSMOS_ATTN_BAD_STRIDE;
+    if (plan_units(d->B, d->S, d->H, d->D).blocks > 0x7FFFFFFF) return COSMOS_ATTN_BAD_SHAPE;
+    return COSMOS_ATTN_OK;
+}
+
+COSMOS_ATTN_API size_t cosmos_norm_rope_bwd_workspace_bytes(const cosmos_norm_rope_bwd_desc* d) {
+    if (validate_norm_rope_bwd(d) != COSMOS_ATTN_OK || !d->dweight) return 0;
+    return (size_t)plan_units(d->B, d->S, d->H, d->D).blocks * d->D * sizeof(float);
+}
+
+COSMOS_ATTN_API int cosmos_norm_rope_bwd(const cosmos_norm_rope_bwd_desc* d, void* workspace, size_t workspace_bytes, void* stream) {
+    const int st = validate_norm_rope_bwd(d);
+    if (st != COSMOS_ATTN_OK) return st;
+    const UnitPlan u = plan_units(d->B, d->S, d->H, d->D);
+    const size_t need = d->dweight ? (size_t)u.blocks * d->D * sizeof(float) : 0;
+    if (need && (!workspace || workspace_bytes < need)) return COSMOS_ATTN_WORKSPACE_TOO_SMALL;
+    if (need && !aligned16(workspace)) return COSMOS_ATTN_BAD_STRIDE;
+    NormRopeBwdParams p;
+    p.x = (const uint16_t*)d->x; p.dy = (const uint16_t*)d->dy; p.dx = (uint16_t*)d->dx;
+    p.weight = d->weight; p.angles = d->angles;
+    p.partials = d->dweight ? (float*)workspace : nullptr;
+    p.x_sb = d->x_stride[0]; p.x_ss = d->x_stride[1]; p.x_sh = d->x_stride[2];
+    p.g_sb = d->dy_stride[0]; p.g_ss = d->dy_stride[1]; p.g_sh = d->dy_stride[2];
+    p.o_sb = d->dx_stride[0]; p.o_ss = d->dx_stride[1]; p.o_sh = d->dx_stride[2];
+    p.B = d->B; p.S = d->S; p.H = d->H; p.D = d->D;
+    p.eps = d->eps;
+    p.heads_per_unit = u.heads_per_unit; p.head_groups = u.head_groups; p.units = u.units;
+    norm_rope_bwd_kernel_t fn = d->dtype == COSMOS_ATTN_BF16 ? pick_bwd<true>(d->D) : pick_bwd<false>(d->D);
+    hipLaunchKernelGGL(fn, dim3((unsigned)u.blocks), dim3(kThreads), 0, (hipStream_t)stream, p);
+    if (hipGetLastError() != hipSuccess) return COSMOS_ATTN_LAUNCH_FAILED;
+    if (d->dweight) {
+        hipLaunchKernelGGL(norm_rope_dweight_kernel, dim3((unsigned)d->D), dim3(kThreads), 0, (hipStream_t)stream,
+                           (const float*)workspace, d->dweight, u.blocks, d->D);
+        if (hipGetLastError() != hipSuccess) return COSMOS_ATTN_LAUNCH_FAILED;
+    }
+    return COSMOS_ATTN_OK;
 }
 
 }  // extern "C"

@@ -12,8 +12,9 @@ with ``backend`` in :361-375 is fixed to the HIP op here.
 layers.  The rule used here is the plain one: linear layers map the tangent with the same weights (primal and tangent
 go through each GEMM stacked along the batch), RMSNorm + RoPE and attention use their fused JVP kernels.
 
-Reverse mode: ``forward`` supports autograd through the projections and the attention kernels only when no gradient
-has to flow through RMSNorm + RoPE, which has no backward kernel; it refuses instead of silently detaching.
+Reverse mode: ``forward`` is differentiable end to end -- the projections through torch, RMSNorm + RoPE through
+``cosmos_norm_rope_bwd`` and the attention through ``cosmos_attn_bwd``.  ``forward_jvp`` runs without autograd (the
+tangent pass of the distillation recipes is taken under ``no_grad``).
 """
 from __future__ import annotations
 
@@ -38,6 +39,24 @@ class HeadRMSNormWeight(nn.Module):
 
     def reset_parameters(self) -> None:
         nn.init.ones_(self.weight)
+
+
+class _NormRopeFn(torch.autograd.Function):
+    """Fused RMSNorm + RoPE with its reverse-mode rule (heads-first output memory, ``[B, S, H, D]`` view)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, rope_emb, eps):
+        y, _ = ops.norm_rope(x, weight, rope_emb, None, eps=eps, out_layout="bhsd")
+        ctx.save_for_backward(x, weight, rope_emb if rope_emb is not None else x.new_empty(0))
+        ctx.has_rope, ctx.eps = rope_emb is not None, eps
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight, rope_emb = ctx.saved_tensors
+        dx, dweight = ops.norm_rope_bwd(x, weight, rope_emb if ctx.has_rope else None, dy, eps=ctx.eps,
+                                        need_dweight=ctx.needs_input_grad[1])
+        return dx, (None if dweight is None else dweight.to(weight.dtype)), None, None
 
 
 class Attention(nn.Module):
@@ -112,21 +131,13 @@ class Attention(nn.Module):
 
     def _norm_rope(self, t, norm: HeadRMSNormWeight, rope_emb, tt=None):
         rope = rope_emb if (self.is_selfattn and rope_emb is not None) else None   # only for self-attention (:409)
+        if tt is None and torch.is_grad_enabled() and (t.requires_grad or norm.weight.requires_grad):
+            return _NormRopeFn.apply(t, norm.weight, rope, norm.eps), None
         return ops.norm_rope(t, norm.weight, rope, tt, eps=norm.eps, out_layout="bhsd")
-
-    def _refuse_reverse_mode(self, *tensors) -> None:
-        if torch.is_grad_enabled() and (
-            any(t is not None and t.requires_grad for t in tensors)
-            or any(p.requires_grad for p in (self.q_proj.weight, self.k_proj.weight, self.q_norm.weight, self.k_norm.weight))
-        ):
-            raise NotImplementedError(
-                "reverse mode through the fused RMSNorm + RoPE is not built: call under torch.no_grad() "
-                "(the attention kernels themselves have a backward, see flash_attention_jvp.attention)")
 
     # ------------------------------------------------------------------ the reference's surface
     def compute_qkv(self, x, context=None, rope_emb=None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         """q, k, v as ``[B, S, H, D]`` (q and k in heads-first memory, ready for the kernels)."""
-        self._refuse_reverse_mode(x, context)
         context = x if context is None else context
         q = self._heads(self.q_proj(x))
         k = self._heads(self.k_proj(context))

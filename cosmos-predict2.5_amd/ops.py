@@ -261,3 +261,56 @@ def norm_rope(
         status = lib.cosmos_norm_rope(ctypes.byref(desc), torch.cuda.current_stream(x.device).cuda_stream)
     _lib.raise_for_status(status)
     return y, ty
+
+
+def norm_rope_bwd(
+    x: torch.Tensor,
+    weight: Optional[torch.Tensor],
+    rope_emb: Optional[torch.Tensor],
+    dy: torch.Tensor,
+    eps: float = 1e-6,
+    need_dweight: bool = True,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Reverse mode of :func:`norm_rope`: ``(dx, dweight)`` from the gradient ``dy`` of its output.  ``x``, ``dy``:
+    ``[B, S, H, D]`` views (any batch / sequence / head strides that are multiples of 8 elements); ``dx`` is contiguous
+    ``[B, S, H, D]``; ``dweight`` is fp32 ``[D]`` (None if not wanted).  This is what autograd derives for the RMSNorm and
+    rotary ops of cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:405-415."""
+    assert x.dim() == 4 and dy.shape == x.shape and dy.dtype == x.dtype and dy.device == x.device
+    B, S, H, D = x.shape
+    assert D in REFERENCE_HEAD_DIMS
+    if D not in SUPPORTED_HEAD_DIMS:
+        raise NotImplementedError(f"head dim {D}: the HIP kernels are built for {SUPPORTED_HEAD_DIMS}")
+    if x.dtype not in _DTYPES:
+        raise NotImplementedError(f"dtype={x.dtype} is not supported (bf16 / fp16)")
+    assert weight is None or weight.shape == (D,)
+    assert rope_emb is None or rope_emb.numel() == S * D, "rope_emb must hold one angle per (position, channel)"
+    if not x.is_cuda:
+        raise RuntimeError("cosmos attention (HIP) needs tensors on a GPU; there is no CPU path")
+    x = x if _kernel_ready(x) else x.contiguous()
+    dy = dy if _kernel_ready(dy) else dy.contiguous()
+    if weight is not None:
+        weight = weight.to(device=x.device, dtype=torch.float32).contiguous()
+    if rope_emb is not None:
+        rope_emb = rope_emb.to(device=x.device, dtype=torch.float32).reshape(S, D).contiguous()
+    dx = torch.empty((B, S, H, D), device=x.device, dtype=x.dtype)
+    dweight = torch.empty((D,), device=x.device, dtype=torch.float32) if need_dweight else None
+
+    desc = _lib.NormRopeBwdDesc()
+    desc.abi_version = _lib.ABI_VERSION
+    desc.dtype = _DTYPES[x.dtype]
+    desc.B, desc.S, desc.H, desc.D = B, S, H, D
+    desc.eps = float(eps)
+    desc.reserved = 0
+    desc.x, desc.dy, desc.dx = x.data_ptr(), dy.data_ptr(), dx.data_ptr()
+    desc.weight = weight.data_ptr() if weight is not None else None
+    desc.angles = rope_emb.data_ptr() if rope_emb is not None else None
+    desc.dweight = dweight.data_ptr() if dweight is not None else None
+    desc.x_stride, desc.dy_stride, desc.dx_stride = _strides3(x), _strides3(dy), _strides3(dx)
+    lib = _lib.load_library()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.cosmos_norm_rope_bwd_workspace_bytes(ctypes.byref(desc))
+        workspace = torch.empty(max(ws_bytes, 16), device=x.device, dtype=torch.uint8)
+        status = lib.cosmos_norm_rope_bwd(ctypes.byref(desc), workspace.data_ptr(), ws_bytes,
+                                          torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.raise_for_status(status)
+    return dx, dweight

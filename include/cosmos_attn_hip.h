@@ -164,6 +164,36 @@ typedef struct cosmos_norm_rope_desc {
 
 COSMOS_ATTN_API int cosmos_norm_rope(const cosmos_norm_rope_desc *desc, void *stream);
 
+/*
+ * Reverse mode of cosmos_norm_rope (what autograd does for the RMSNorm and rotary ops of networks/minimal_v4_dit.py:405-415
+ * during training): from dy = dL/dy,
+ *     dn = R^T dy                      (rotation by the negated angles; RMSNorm's 16-bit rounding is passed straight through)
+ *     dx = r (weight * dn) - x r^3 mean_d(x * weight * dn),      r = rsqrt(mean_d(x^2) + eps)
+ *     dweight[j] = sum over all (b, s, h) of dn[j] x[j] r        (fp32, optional)
+ * x, dy, dx: [B, S, H, D] through their own (batch, sequence, head) element strides.  dweight needs a workspace of
+ * cosmos_norm_rope_bwd_workspace_bytes(desc) bytes (per-block partial sums, added in a fixed order: results are
+ * bitwise reproducible); with dweight == NULL no workspace is needed.  Two launches (one without dweight).
+ */
+typedef struct cosmos_norm_rope_bwd_desc {
+    int32_t abi_version;     /* COSMOS_ATTN_ABI_VERSION */
+    int32_t dtype;           /* element type of x, dy, dx */
+    int32_t B, S, H, D;
+    float eps;
+    int32_t reserved;        /* 0 */
+    const void *x, *dy;      /* device */
+    const float *weight;     /* [D] fp32 or NULL = ones */
+    const float *angles;     /* [S, D] fp32 or NULL = no rotation */
+    void *dx;                /* device */
+    float *dweight;          /* [D] fp32, device; NULL = not wanted */
+    int64_t x_stride[3];
+    int64_t dy_stride[3];
+    int64_t dx_stride[3];
+} cosmos_norm_rope_bwd_desc;
+
+COSMOS_ATTN_API size_t cosmos_norm_rope_bwd_workspace_bytes(const cosmos_norm_rope_bwd_desc *desc);
+COSMOS_ATTN_API int cosmos_norm_rope_bwd(const cosmos_norm_rope_bwd_desc *desc, void *workspace, size_t workspace_bytes,
+                                         void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -27,12 +27,15 @@ Functions
                             ``torch.func.jvp`` -- the oracle the tolerance is quoted against.
 ``norm_rope_closed_form``   numpy fp64 closed form of value and tangent, independent of autograd; optional
                             16-bit rounding of the normalised tensor (RMSNorm's output type).
+``norm_rope_grads_torch``   torch autograd (reverse mode) of the same function: (dx, dweight) for a cotangent dy.
+``norm_rope_grads_closed_form``  numpy fp64 closed form of the reverse mode.
 
-Parity status: the mathematics is pinned in ``tests/test_oracle.py`` (closed form against torch forward AD
+Parity status: the mathematics is pinned in ``tests/test_oracle_norm_rope.py`` (closed form against torch forward AD
 and torch's own ``rms_norm``, finite differences, brute-force scalar loops, rotation invariants: zero angle,
 pair-norm preservation, angle additivity, relative-position property; RMSNorm invariants: scale invariance
-and the zero tangent along x).  Against Transformer Engine's binaries themselves -- in particular the exact
-rounding points of its fused kernels -- PARITY UNPINNED: the library is absent and the reference holds no
+and the zero tangent along x; the reverse mode against torch autograd, the adjoint identity <dy, J tx> = <J^T dy, tx>
+with the pinned forward-mode closed form as J, and finite differences in the weight).  Against Transformer Engine's
+binaries themselves -- in particular the exact rounding points of its fused kernels -- PARITY UNPINNED: the library is absent and the reference holds no
 stored outputs of this step.
 """
 from __future__ import annotations
@@ -103,6 +106,44 @@ def norm_rope_torch(x, weight=None, angles=None, tx=None, eps: float = 1e-6):
     tx = torch.as_tensor(np.asarray(tx, dtype=np.float32)) if not isinstance(tx, torch.Tensor) else tx.detach().float().cpu()
     y, ty = torch.func.jvp(f, (x,), (tx,))
     return y, ty
+
+
+def norm_rope_grads_closed_form(x, weight=None, angles=None, dy=None, eps: float = 1e-6):
+    """numpy fp64 reverse mode: (dx, dweight) with dy the cotangent of y.
+        dn = R^T dy,   dx = r (g dn) - x r^3 mean(x g dn),   dweight = sum_rows dn x r."""
+    x = np.asarray(x, dtype=np.float64)
+    dy = np.asarray(dy, dtype=np.float64)
+    B, S, H, D = x.shape
+    g = np.ones(D) if weight is None else np.asarray(weight, dtype=np.float64)
+    if angles is None:
+        dn = dy
+    else:
+        a = np.asarray(angles, dtype=np.float64).reshape(1, S, 1, D)
+        # y = n cos(a) + rotate_half(n) sin(a);  the adjoint of rotate_half is its negative
+        dn = dy * np.cos(a) - _rotate_half_np(dy * np.sin(a))
+    r = 1.0 / np.sqrt((x * x).mean(axis=-1, keepdims=True) + eps)
+    gdn = g * dn
+    dx = r * gdn - x * r**3 * (x * gdn).mean(axis=-1, keepdims=True)
+    dweight = (dn * x * r).sum(axis=(0, 1, 2))
+    return dx, dweight
+
+
+def norm_rope_grads_torch(x, weight=None, angles=None, dy=None, eps: float = 1e-6, dtype=None):
+    """torch autograd of rms_norm + rotate-half rotation: (dx, dweight) for the cotangent dy (fp32 unless ``dtype``)."""
+    import torch
+    import torch.nn.functional as F
+
+    dt = dtype or torch.float32
+    t = lambda z: torch.as_tensor(np.asarray(z)).to(dt) if not isinstance(z, torch.Tensor) else z.detach().cpu().to(dt)
+    x = t(x).requires_grad_(True)
+    B, S, H, D = x.shape
+    w = (torch.ones(D, dtype=dt) if weight is None else t(weight)).requires_grad_(True)
+    n = F.rms_norm(x, (D,), weight=w, eps=eps)
+    if angles is not None:
+        a = t(angles).reshape(1, S, 1, D)
+        n = n * torch.cos(a) + torch.cat([-n[..., D // 2:], n[..., : D // 2]], dim=-1) * torch.sin(a)
+    dx, dw = torch.autograd.grad(n, (x, w), grad_outputs=t(dy))
+    return dx, dw
 
 
 def rope_angles_3d(T: int, Hh: int, W: int, D: int, theta: float = 10000.0) -> np.ndarray:

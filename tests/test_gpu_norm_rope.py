@@ -204,3 +204,82 @@ def test_feeds_the_attention_kernel_without_a_transpose(pkg, oracle, nr_oracle, 
         ma, rl = oracle.error_metrics(got.float().cpu(), want)
         print(f"  {name}: max_abs={ma:.3e} rel_l2={rl:.3e}", flush=True)
         assert ma <= 2e-2 and rl <= 1e-2
+
+
+# ---------------------------------------------------------------------------------------------- reverse mode
+def check_grad(name, got, want, max_abs=MAX_ABS, rel_l2=REL_L2):
+    got = got.float().cpu().double().numpy()
+    ma = float(np.abs(got - want).max())
+    rl = float(np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30))
+    lim = max_abs * max(1.0, float(np.abs(want).max()))
+    print(f"  {name}: max_abs={ma:.3e} (limit {lim:.3e}) rel_l2={rl:.3e}", flush=True)
+    assert math.isfinite(ma) and ma <= lim, f"{name}: max-abs {ma} > {lim}"
+    assert rl <= rel_l2, f"{name}: rel-L2 {rl} > {rel_l2}"
+
+
+def run_bwd_case(pkg, nr_oracle, gpu, B, S, H, D, dtype=torch.bfloat16, rope=True, weight=True, seed=0, dy_layout="bshd",
+                 need_dweight=True):
+    print(f"norm_rope_bwd case B={B} S={S} H={H} D={D} {dtype} rope={rope} weight={weight} dy_layout={dy_layout} seed={seed}", flush=True)
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, S, H, D, generator=g).to(dtype)
+    dy = torch.randn(B, S, H, D, generator=g).to(dtype)
+    w = (1.0 + 0.2 * torch.randn(D, generator=g)) if weight else None
+    a = torch.from_numpy(nr_oracle.rope_angles_3d(1, 1, S, D)) if rope else None
+    dyd = dy.to(gpu)
+    if dy_layout == "bhsd":     # the gradient as the attention backward hands it over: heads-first memory
+        dyd = dyd.transpose(1, 2).contiguous().transpose(1, 2)
+    dx, dw = pkg.norm_rope_bwd(x.to(gpu), None if w is None else w.to(gpu), None if a is None else a.to(gpu), dyd,
+                               need_dweight=need_dweight)
+    torch.cuda.synchronize()
+    assert dx.shape == x.shape and dx.dtype == dtype and dx.is_contiguous()
+    want_dx, want_dw = nr_oracle.norm_rope_grads_closed_form(x.float().numpy(), None if w is None else w.numpy(),
+                                                             None if a is None else a.numpy(), dy.float().numpy())
+    check_grad("dx", dx, want_dx)
+    if need_dweight:
+        assert dw.dtype == torch.float32 and dw.shape == (D,)
+        check_grad("dweight", dw, want_dw, rel_l2=2e-3)     # fp32 sums of products of 16-bit inputs
+    else:
+        assert dw is None
+    return dx, dw
+
+
+@pytest.mark.parametrize("D", [16, 32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_bwd_head_dims_and_dtypes(pkg, nr_oracle, gpu, D, dtype):
+    run_bwd_case(pkg, nr_oracle, gpu, 2, 37, 3, D, dtype=dtype, seed=D)
+
+
+@pytest.mark.parametrize("H", [1, 3, 4, 5, 16])
+@pytest.mark.parametrize("S", [1, 17, 300])
+def test_bwd_ragged_sizes(pkg, nr_oracle, gpu, H, S):
+    run_bwd_case(pkg, nr_oracle, gpu, 1, S, H, 128, seed=H * 1000 + S)
+
+
+@pytest.mark.parametrize("rope,weight", [(False, True), (True, False), (False, False)])
+def test_bwd_optional_operands(pkg, nr_oracle, gpu, rope, weight):
+    run_bwd_case(pkg, nr_oracle, gpu, 1, 50, 4, 64, rope=rope, weight=weight, seed=5)
+
+
+def test_bwd_strided_gradient_no_dweight_and_determinism(pkg, nr_oracle, gpu):
+    a, wa = run_bwd_case(pkg, nr_oracle, gpu, 2, 130, 6, 128, dy_layout="bhsd", seed=6)
+    b, wb = run_bwd_case(pkg, nr_oracle, gpu, 2, 130, 6, 128, dy_layout="bshd", seed=6)
+    assert torch.equal(a, b) and torch.equal(wa, wb)            # same values through either gradient layout, bit for bit
+    c, _ = run_bwd_case(pkg, nr_oracle, gpu, 2, 130, 6, 128, seed=6, need_dweight=False)
+    assert torch.equal(a, c)
+
+
+def test_bwd_many_blocks_dweight_reduction(pkg, nr_oracle, gpu):
+    """Enough rows for thousands of partial-sum rows: the two-stage dweight reduction against the oracle."""
+    run_bwd_case(pkg, nr_oracle, gpu, 1, 20000, 16, 128, seed=8)
+
+
+def test_autograd_through_norm_rope_matches_the_raw_op(pkg, nr_oracle, gpu):
+    torch.manual_seed(0)
+    m = pkg.Attention(256, None, n_heads=2, head_dim=128).to(device=gpu, dtype=torch.bfloat16)
+    x = torch.randn(1, 40, 2, 128, device=gpu, dtype=torch.bfloat16, requires_grad=True)
+    a = torch.from_numpy(nr_oracle.rope_angles_3d(1, 1, 40, 128)).to(gpu)
+    y, _ = m._norm_rope(x, m.q_norm, a)
+    dy = torch.randn_like(y)
+    y.backward(dy)
+    dx, dw = pkg.norm_rope_bwd(x.detach(), m.q_norm.weight.detach(), a, dy)
+    assert torch.equal(x.grad, dx) and torch.equal(m.q_norm.weight.grad, dw.to(torch.bfloat16))

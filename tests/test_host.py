@@ -176,6 +176,43 @@ def test_norm_rope_desc_layout_and_status_codes(pkg):
         assert got == want, (over, got)
 
 
+def test_norm_rope_bwd_desc_layout_and_status_codes(pkg):
+    L, lib = pkg._lib, pkg._lib.load_library()
+    # 8 x int32/float, 6 pointers, 3 x 3 int64
+    assert ctypes.sizeof(L.NormRopeBwdDesc) == 32 + 6 * 8 + 3 * 3 * 8
+    assert L.NormRopeBwdDesc.x.offset == 32 and L.NormRopeBwdDesc.dx_stride.offset == 32 + 6 * 8 + 2 * 3 * 8
+
+    def desc(**over):
+        D = L.NormRopeBwdDesc()
+        D.abi_version, D.dtype, D.B, D.S, D.H, D.D, D.eps = L.ABI_VERSION, L.DTYPE_BF16, 2, 100, 6, 64, 1e-6
+        D.x, D.dy, D.dx, D.dweight = 0x7F0000000000, 0x7F0000100000, 0x7F0000200000, 0x7F0000300000   # never dereferenced
+        D.x_stride = D.dy_stride = D.dx_stride = (ctypes.c_int64 * 3)(100 * 6 * 64, 6 * 64, 64)
+        for k, v in over.items():
+            setattr(D, k, v)
+        return D
+
+    ws = lambda D: lib.cosmos_norm_rope_bwd_workspace_bytes(ctypes.byref(D))
+    run = lambda D: lib.cosmos_norm_rope_bwd(ctypes.byref(D), None, 0, None)
+    # 2 x 100 positions x 2 groups of 4 heads = 400 thread groups, 32 per block (8 threads per row of 64) -> 13 blocks x 64 floats
+    assert ws(desc()) == 13 * 64 * 4
+    assert ws(desc(dweight=None)) == 0
+    assert run(desc()) == L.ST_WORKSPACE
+    cases = [
+        (dict(abi_version=1), L.ST_BAD_ARG),
+        (dict(H=0), L.ST_BAD_ARG),
+        (dict(dy=None), L.ST_BAD_ARG),
+        (dict(dtype=5), L.ST_UNSUPPORTED),
+        (dict(D=256), L.ST_UNSUPPORTED),
+        (dict(D=24), L.ST_BAD_SHAPE),
+        (dict(dx=0x7F0000200008), L.ST_BAD_STRIDE),
+        (dict(dy_stride=(ctypes.c_int64 * 3)(100 * 6 * 66, 6 * 66, 66)), L.ST_BAD_STRIDE),
+    ]
+    for over, want in cases:
+        D = desc(**over)
+        assert ws(D) == 0, over
+        assert run(D) == want, (over, run(D))
+
+
 def test_norm_rope_argument_checks(pkg):
     x = torch.zeros(1, 8, 2, 64, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="GPU"):                   # no CPU path, no fallback

@@ -76,3 +76,27 @@ def test_rope_is_skipped_for_cross_attention(dit_oracle):
     o1, _ = dit_oracle.attention_module_torch(w, x, c, a, H, D, dtype=torch.float64)
     o2, _ = dit_oracle.attention_module_torch(w, x, c, None, H, D, dtype=torch.float64)
     assert torch.equal(o1, o2)
+
+
+def test_module_grads_adjoint_identity_and_weight_finite_differences(dit_oracle):
+    B, Mq, K, H, D = 1, 9, 16, 2, 16
+    g = torch.Generator().manual_seed(21)
+    r = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    w = make_weights(K, K, H, D, 22)
+    x, tx, dout = r(B, Mq, K), r(B, Mq, K), r(B, Mq, K)
+    half = np.random.default_rng(23).standard_normal((Mq, D // 2))
+    angles = np.concatenate([half, half], -1)
+    grads = dit_oracle.attention_module_grads_torch(w, x, dout, None, angles, H, D, dtype=torch.float64)
+    # <dout, J tx> = <J^T dout, tx> with J from forward mode (pinned above)
+    _, tout = dit_oracle.attention_module_torch(w, x, None, angles, H, D, tx, dtype=torch.float64)
+    assert abs(float((dout * tout).sum()) - float((grads["x"] * tx).sum())) < 1e-9
+    # one random direction in every weight, central differences of <dout, out>
+    h = 1e-6
+    for name in w:
+        dirw = r(*w[name].shape)
+        wp, wm = dict(w), dict(w)
+        wp[name], wm[name] = w[name] + h * dirw, w[name] - h * dirw
+        fp = dit_oracle.attention_module_torch(wp, x, None, angles, H, D, dtype=torch.float64)[0]
+        fm = dit_oracle.attention_module_torch(wm, x, None, angles, H, D, dtype=torch.float64)[0]
+        fd = float((dout * (fp - fm)).sum()) / (2 * h)
+        assert abs(fd - float((grads[name] * dirw).sum())) < 1e-6, name

@@ -78,6 +78,16 @@ def test_rotation_invariants(nr_oracle):
     np.testing.assert_allclose((n0 ** 2).mean(-1), 1.0, atol=1e-12)
 
 
+def test_angle_additivity(nr_oracle):
+    """Turning by a and then by b is turning by a + b (rows of mean square 1 pass the second RMSNorm unchanged at eps = 0)."""
+    S, D = 4, 32
+    x, a, b = rnd((1, S, 2, D), 24), paired_angles(S, D, 25), paired_angles(S, D, 26)
+    y1, _ = nr_oracle.norm_rope_closed_form(x, None, a, eps=0.0)
+    y2, _ = nr_oracle.norm_rope_closed_form(y1, None, b, eps=0.0)
+    y12, _ = nr_oracle.norm_rope_closed_form(x, None, a + b, eps=0.0)
+    np.testing.assert_allclose(y2, y12, atol=1e-12)
+
+
 def test_relative_position_property(nr_oracle):
     """<rope(q, m), rope(k, n)> depends on m - n only: angles m * f and n * f for one frequency vector f."""
     D, H = 32, 1
@@ -135,3 +145,35 @@ def test_angle_layout_matches_reference_construction(nr_oracle):
     assert np.array_equal(a4[0, 0, 3, dim_t // 2 + dim_h // 2 : D // 2], a4[1, 2, 3, dim_t // 2 + dim_h // 2 : D // 2])
     # first frequency of every block is 1: the angle equals the coordinate
     assert a4[1, 2, 3, 0] == 1 and a4[1, 2, 3, dim_t // 2] == 2 and a4[1, 2, 3, dim_t // 2 + dim_h // 2] == 3
+
+
+# ---------------------------------------------------------------- reverse mode
+@pytest.mark.parametrize("B,S,H,D", [(1, 5, 3, 16), (2, 4, 2, 64)])
+@pytest.mark.parametrize("rope", [True, False])
+def test_grads_closed_form_matches_torch_autograd(nr_oracle, B, S, H, D, rope):
+    x, dy, w = rnd((B, S, H, D), 31), rnd((B, S, H, D), 32), 1.0 + 0.2 * rnd((D,), 33)
+    a = rnd((S, D), 34, 2.0) if rope else None        # arbitrary angles: the two members of a pair may differ
+    dx, dw = nr_oracle.norm_rope_grads_closed_form(x, w, a, dy)
+    dxt, dwt = nr_oracle.norm_rope_grads_torch(x, w, a, dy, dtype=torch.float64)
+    np.testing.assert_allclose(dx, dxt.numpy(), atol=1e-12)
+    np.testing.assert_allclose(dw, dwt.numpy(), atol=1e-12)
+
+
+def test_grads_adjoint_identity_with_the_pinned_jvp(nr_oracle):
+    """<dy, J tx> = <J^T dy, tx>, J from the forward-mode closed form pinned above."""
+    B, S, H, D = 2, 6, 3, 32
+    x, tx, dy, w, a = rnd((B, S, H, D), 35), rnd((B, S, H, D), 36), rnd((B, S, H, D), 37), 1.0 + 0.2 * rnd((D,), 38), paired_angles(S, D, 39)
+    _, ty = nr_oracle.norm_rope_closed_form(x, w, a, tx)
+    dx, _ = nr_oracle.norm_rope_grads_closed_form(x, w, a, dy)
+    assert abs(float((dy * ty).sum()) - float((dx * tx).sum())) < 1e-10
+
+
+def test_dweight_matches_finite_differences(nr_oracle):
+    B, S, H, D = 1, 5, 2, 16
+    x, dy, w, a = rnd((B, S, H, D), 40), rnd((B, S, H, D), 41), 1.0 + 0.2 * rnd((D,), 42), paired_angles(S, D, 43)
+    _, dw = nr_oracle.norm_rope_grads_closed_form(x, w, a, dy)
+    dirw = rnd((D,), 44)
+    h = 1e-6
+    yp, _ = nr_oracle.norm_rope_closed_form(x, w + h * dirw, a)
+    ym, _ = nr_oracle.norm_rope_closed_form(x, w - h * dirw, a)
+    assert abs(float((dy * (yp - ym)).sum()) / (2 * h) - float((dw * dirw).sum())) < 1e-7
