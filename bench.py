@@ -1,6 +1,6 @@
 """Benchmark of the attention forward + JVP hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk|dblk] [--no-cpu]
 
 A "step" is one call of the hot path (re-tiling kernel + attention kernel, through the Python host and
 the C ABI) over one batch of synthetic tensors that are already resident in HBM.  Default workload: the
@@ -50,6 +50,8 @@ WORKLOADS = {
     # the whole DiT self-attention module with a tangent: 4 projections (library GEMMs on stacked primal + tangent),
     # RMSNorm + RoPE (+ tangent) of q and k, attention forward + JVP
     "blk": ("2B DiT self-attention module fwd+JVP bf16 720p B1 L84480 K2048 H16 d128", 1, 16, 84480, 84480, 128, "module", False, False),
+    # one whole DiT block with a tangent: adaLN modulation, self-attention, text cross-attention, MLP, gated residuals
+    "dblk": ("2B DiT block fwd+JVP bf16 720p B1 T24 H44 W80 D2048 heads16 text512x1024 adaLN-LoRA256", 1, 16, 84480, 512, 128, "block", False, False),
 }
 PEAK_HBM_GBS = 8000.0
 
@@ -210,6 +212,63 @@ def bench_module(args, pkg, dev, desc_txt, B, H, L, D):
     print(json.dumps(result), flush=True)
 
 
+def bench_block(args, pkg, dev, desc_txt, B, H, L, Mk, D):
+    """One step = Block.forward_jvp of the 2B DiT's transformer block at the 720p token grid."""
+    nro = entry.load_norm_rope_oracle()
+    K, Kc, T, Hh, W = H * D, 1024, 24, 44, 80
+    assert T * Hh * W == L
+    torch.manual_seed(0)
+    m = pkg.Block(K, Kc, H, mlp_ratio=4.0, use_adaln_lora=True, adaln_lora_dim=256)
+    m.init_weights()
+    with torch.no_grad():   # a freshly initialised block has zero gates; give the modulation something to do
+        for mod in (m.adaln_modulation_self_attn, m.adaln_modulation_cross_attn, m.adaln_modulation_mlp):
+            mod[-1].weight.copy_(torch.randn_like(mod[-1].weight) / 16.0)
+    m = m.to(device=dev, dtype=torch.bfloat16).eval()
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(s, generator=g, device=dev)
+    x, tx = rn(B, T, Hh, W, K).bfloat16(), (0.1 * rn(B, T, Hh, W, K)).bfloat16()
+    emb, temb = rn(B, T, K).bfloat16(), (0.1 * rn(B, T, K)).bfloat16()
+    lora, tlora = (0.3 * rn(B, T, 3 * K)).bfloat16(), (0.03 * rn(B, T, 3 * K)).bfloat16()
+    ctx = rn(B, Mk, Kc).bfloat16()
+    rope = torch.from_numpy(nro.rope_angles_3d(T, Hh, W, D)).to(dev).reshape(L, 1, 1, D)
+    gemm = lambda rows, k, n: 2.0 * rows * k * n
+    flops = {
+        "self_attn_projections": 4 * 2 * gemm(B * L, K, K),
+        "self_attn": 6 * 2.0 * B * H * L * L * D,
+        "cross_attn_projections": 2 * 2 * gemm(B * L, K, K) + 2 * gemm(B * Mk, Kc, K),
+        "cross_attn": 4 * 2.0 * B * H * L * Mk * D,
+        "mlp": 2 * 2 * gemm(B * L, K, 4 * K),
+    }
+    total = sum(flops.values())
+    step = lambda: m.forward_jvp(x, tx, emb, temb, ctx, rope, lora, tlora)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        out = step()
+    e1.record()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / args.steps
+    avg = e0.elapsed_time(e1) / args.steps
+    del out
+    achieved = total / (avg * 1e-3) / 1e12
+    result = {
+        "metric": "DiT block fwd+JVP TFLOP/s & % bf16 MFMA peak @ 2B 720p (L=84480); ms per call",
+        "value": total / sec / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": desc_txt, "flop_per_call": total, "flop_parts": flops,
+                   "pct_of_bf16_mfma_peak": 100.0 * total / sec / 1e12 / PEAK_BF16_TFLOPS},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "whole block call (attn_fwd_jvp_kernel dominates)", "kernel_ms_avg": avg},
+    }
+    print(json.dumps(result), flush=True)
+
+
 def copy_calibration(dev):
     """One plain elementwise copy kernel that reads 1 GiB and writes 1 GiB: the known-size launch the FETCH_SIZE /
     WRITE_SIZE counters are scaled by."""
@@ -307,6 +366,8 @@ def main():
     desc_txt, B, H, Lq, Lkv, d, tangents, rms, padded = WORKLOADS[args.workload]
     if tangents == "bwd":
         return bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
+    if tangents == "block":
+        return bench_block(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
     if tangents == "module":
         return bench_module(args, pkg, dev, desc_txt, B, H, Lq, d)
     if tangents in ("norm_rope", "norm_rope_bwd"):

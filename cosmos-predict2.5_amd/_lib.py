@@ -134,6 +134,44 @@ class NormRopeBwdDesc(ctypes.Structure):
     ]
 
 
+class LnModulateDesc(ctypes.Structure):
+    """Mirror of ``struct cosmos_ln_modulate_desc``."""
+
+    _fields_ = [
+        ("abi_version", ctypes.c_int32), ("dtype", ctypes.c_int32),
+        ("D", ctypes.c_int32), ("rows_per_group", ctypes.c_int32),
+        ("eps", ctypes.c_float), ("reserved", ctypes.c_int32),
+        ("rows", ctypes.c_int64),
+        ("x", ctypes.c_void_p), ("tx", ctypes.c_void_p),
+        ("shift", ctypes.c_void_p), ("scale", ctypes.c_void_p),
+        ("tshift", ctypes.c_void_p), ("tscale", ctypes.c_void_p),
+        ("y", ctypes.c_void_p), ("ty", ctypes.c_void_p),
+    ]
+
+
+class GatedResidualDesc(ctypes.Structure):
+    """Mirror of ``struct cosmos_gated_residual_desc``."""
+
+    _fields_ = [
+        ("abi_version", ctypes.c_int32), ("dtype", ctypes.c_int32),
+        ("D", ctypes.c_int32), ("rows_per_group", ctypes.c_int32),
+        ("rows", ctypes.c_int64),
+        ("x", ctypes.c_void_p), ("tx", ctypes.c_void_p), ("res", ctypes.c_void_p), ("tres", ctypes.c_void_p),
+        ("gate", ctypes.c_void_p), ("tgate", ctypes.c_void_p),
+        ("out", ctypes.c_void_p), ("tout", ctypes.c_void_p),
+    ]
+
+
+class GeluDesc(ctypes.Structure):
+    """Mirror of ``struct cosmos_gelu_desc``."""
+
+    _fields_ = [
+        ("abi_version", ctypes.c_int32), ("dtype", ctypes.c_int32),
+        ("n", ctypes.c_int64),
+        ("h", ctypes.c_void_p), ("th", ctypes.c_void_p), ("a", ctypes.c_void_p), ("ta", ctypes.c_void_p),
+    ]
+
+
 EXPORTS = {
     "cosmos_attn_abi_version": (ctypes.c_int, []),
     "cosmos_attn_status_string": (ctypes.c_char_p, [ctypes.c_int]),
@@ -146,6 +184,9 @@ EXPORTS = {
     "cosmos_norm_rope": (ctypes.c_int, [ctypes.POINTER(NormRopeDesc), ctypes.c_void_p]),
     "cosmos_norm_rope_bwd_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(NormRopeBwdDesc)]),
     "cosmos_norm_rope_bwd": (ctypes.c_int, [ctypes.POINTER(NormRopeBwdDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "cosmos_ln_modulate": (ctypes.c_int, [ctypes.POINTER(LnModulateDesc), ctypes.c_void_p]),
+    "cosmos_gated_residual": (ctypes.c_int, [ctypes.POINTER(GatedResidualDesc), ctypes.c_void_p]),
+    "cosmos_gelu": (ctypes.c_int, [ctypes.POINTER(GeluDesc), ctypes.c_void_p]),
 }
 
 _lib = None

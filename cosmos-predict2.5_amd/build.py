@@ -14,7 +14,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_ROOT = os.path.dirname(PKG_DIR)
 LIB_NAME = "libcosmos_attn_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
-SOURCES = [os.path.join(PKG_DIR, "csrc", name) for name in ("attn_fwd_jvp_gfx950.hip", "attn_bwd_gfx950.hip", "norm_rope_gfx950.hip")]
+SOURCES = [os.path.join(PKG_DIR, "csrc", name) for name in ("attn_fwd_jvp_gfx950.hip", "attn_bwd_gfx950.hip", "norm_rope_gfx950.hip", "block_elementwise_gfx950.hip")]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

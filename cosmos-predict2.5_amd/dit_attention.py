@@ -118,8 +118,12 @@ class Attention(nn.Module):
 
     @staticmethod
     def _stack(x: torch.Tensor, tx: Optional[torch.Tensor]):
-        """Primal and tangent along the batch, so that a linear layer maps both in one GEMM."""
-        return x if tx is None else torch.cat([x, tx], dim=0)
+        """Primal and tangent along the batch, so that a linear layer maps both in one GEMM (no copy when the two
+        already are the halves of one buffer)."""
+        if tx is None:
+            return x
+        both = ops.as_stacked(x, tx)
+        return both if both is not None else torch.cat([x, tx], dim=0)
 
     @staticmethod
     def _apply_stacked(lin: nn.Linear, xs: torch.Tensor, has_tangent: bool):

@@ -1,0 +1,228 @@
+"""The DiT transformer ``Block`` (self-attention, cross-attention and MLP, each behind a LayerNorm with adaLN
+modulation and a gated residual) on the HIP attention path, with a forward that also carries a tangent.
+
+Reference: ``Block`` (cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:993-1242) and ``GPT2FeedForward``
+(:222-249) -- same constructor arguments, sub-module and parameter names (``self_attn.*``, ``cross_attn.*``,
+``mlp.layer1/2.weight``, ``adaln_modulation_{self_attn,cross_attn,mlp}.{1,2}.weight``: a reference state dict of the
+block loads as is), ``init_weights``, ``forward(x_B_T_H_W_D, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D,
+adaln_lora_B_T_3D, extra_per_block_pos_emb)``.
+
+``forward_jvp`` pushes a tangent of ``(x, emb, adaln_lora)`` through the block: what a consistency-distillation step
+needs when it differentiates the network along (x_t, t).  The reference ships the attention JVP kernel but no caller
+that does this, so the rules are written out here: LayerNorm + modulation, GELU and the gated residuals each in one
+fused HIP pass (fp32 arithmetic on 16-bit tensors), the tiny modulation MLP by torch forward AD, linear layers on
+primal and tangent stacked in one GEMM (the fused passes write both into one buffer, so nothing is copied to stack
+them), attention through ``Attention.forward_jvp``.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+from torch import nn
+
+from . import ops
+from .dit_attention import Attention
+
+
+class GPT2FeedForward(nn.Module):
+    def __init__(self, d_model: int, d_ff: int):
+        super().__init__()
+        self.activation = nn.GELU()
+        self.layer1 = nn.Linear(d_model, d_ff, bias=False)
+        self.layer2 = nn.Linear(d_ff, d_model, bias=False)
+        self._layer_id = None
+        self._dim = d_model
+        self._hidden_dim = d_ff
+        self.init_weights()
+
+    def init_weights(self) -> None:
+        """minimal_v4_dit.py:234-242: truncated normal, std 1/sqrt(fan_in), the second layer scaled down with depth."""
+        std = 1.0 / math.sqrt(self._dim)
+        torch.nn.init.trunc_normal_(self.layer1.weight, std=std, a=-3 * std, b=3 * std)
+        std = 1.0 / math.sqrt(self._hidden_dim)
+        if self._layer_id is not None:
+            std = std / math.sqrt(2 * (self._layer_id + 1))
+        torch.nn.init.trunc_normal_(self.layer2.weight, std=std, a=-3 * std, b=3 * std)
+
+    def forward(self, x: torch.Tensor):
+        return self.layer2(self.activation(self.layer1(x)))
+
+    @torch.no_grad()
+    def forward_jvp(self, x: torch.Tensor, tx: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        b = x.shape[0]
+        both = ops.as_stacked(x, tx)
+        h = self.layer1(both if both is not None else torch.cat([x, tx], dim=0))
+        ops.gelu(h[:b], h[b:], inplace=True)       # a = gelu(h), ta = th gelu'(h), in place on the stacked buffer
+        y = self.layer2(h)
+        return y[:b], y[b:]
+
+
+class Block(nn.Module):
+    def __init__(
+        self,
+        x_dim: int,
+        context_dim: int,
+        num_heads: int,
+        mlp_ratio: float = 4.0,
+        use_adaln_lora: bool = False,
+        adaln_lora_dim: int = 256,
+        backend: str = "hip",
+        image_context_dim: Optional[int] = None,
+        use_wan_fp32_strategy: bool = False,
+    ):
+        super().__init__()
+        if image_context_dim is not None:
+            raise NotImplementedError("the image-conditioned cross-attention (I2VCrossAttention) is not built")
+        if use_wan_fp32_strategy:
+            raise NotImplementedError("use_wan_fp32_strategy is not built")
+        self.x_dim = x_dim
+        self.layer_norm_self_attn = nn.LayerNorm(x_dim, elementwise_affine=False, eps=1e-6)
+        self.self_attn = Attention(x_dim, None, num_heads, x_dim // num_heads, qkv_format="bshd", backend=backend)
+        self.layer_norm_cross_attn = nn.LayerNorm(x_dim, elementwise_affine=False, eps=1e-6)
+        self.cross_attn = Attention(x_dim, context_dim, num_heads, x_dim // num_heads, qkv_format="bshd", backend=backend)
+        self.layer_norm_mlp = nn.LayerNorm(x_dim, elementwise_affine=False, eps=1e-6)
+        self.mlp = GPT2FeedForward(x_dim, int(x_dim * mlp_ratio))
+
+        self.use_adaln_lora = use_adaln_lora
+
+        def modulation():
+            if use_adaln_lora:
+                return nn.Sequential(nn.SiLU(), nn.Linear(x_dim, adaln_lora_dim, bias=False),
+                                     nn.Linear(adaln_lora_dim, 3 * x_dim, bias=False))
+            return nn.Sequential(nn.SiLU(), nn.Linear(x_dim, 3 * x_dim, bias=False))
+
+        self.adaln_modulation_self_attn = modulation()
+        self.adaln_modulation_cross_attn = modulation()
+        self.adaln_modulation_mlp = modulation()
+        self.cp_size = None
+        self.use_wan_fp32_strategy = use_wan_fp32_strategy
+
+    def set_context_parallel_group(self, process_group, ranks, stream):
+        self.cp_size = None if ranks is None else len(ranks)
+        self.self_attn.set_context_parallel_group(process_group=process_group, ranks=ranks, stream=stream)
+
+    def reset_parameters(self) -> None:
+        """minimal_v4_dit.py:1095-1111: the last modulation layer starts at zero (the block starts as the identity)."""
+        mods = (self.adaln_modulation_self_attn, self.adaln_modulation_cross_attn, self.adaln_modulation_mlp)
+        if self.use_adaln_lora:
+            std = 1.0 / math.sqrt(self.x_dim)
+            for m in mods:
+                torch.nn.init.trunc_normal_(m[1].weight, std=std, a=-3 * std, b=3 * std)
+                torch.nn.init.zeros_(m[2].weight)
+        else:
+            for m in mods:
+                torch.nn.init.zeros_(m[1].weight)
+
+    def init_weights(self) -> None:
+        self.reset_parameters()
+        self.self_attn.init_weights()
+        self.cross_attn.init_weights()
+        self.mlp.init_weights()
+
+    # ------------------------------------------------------------------ pieces
+    def _modulation(self, mod: nn.Sequential, emb_B_T_D, adaln_lora_B_T_3D, like):
+        """(shift, scale, gate), each ``[B, T, 1, 1, D]`` in the type of x (minimal_v4_dit.py:1131-1162)."""
+        m = mod(emb_B_T_D)
+        if self.use_adaln_lora:
+            m = m + adaln_lora_B_T_3D
+        return tuple(c[:, :, None, None, :].type_as(like) for c in m.chunk(3, dim=-1))
+
+    def _modulation_jvp(self, mod: nn.Sequential, emb, temb, lora, tlora, like):
+        """Modulation and its tangent; the tensors are ``[B, T, 3 D]``, tiny next to x: forward AD does it."""
+        f = (lambda e, l: mod(e) + l) if self.use_adaln_lora else (lambda e, l: mod(e))
+        if lora is None:
+            lora = emb.new_zeros(())
+        temb = torch.zeros_like(emb) if temb is None else temb
+        tlora = torch.zeros_like(lora) if tlora is None else tlora
+        m, tm = torch.func.jvp(f, (emb, lora), (temb, tlora))
+        cut = lambda z: tuple(c[:, :, None, None, :].type_as(like) for c in z.chunk(3, dim=-1))
+        return cut(m), cut(tm)
+
+    @staticmethod
+    def _modulate(norm_layer, x, scale, shift):
+        return norm_layer(x) * (1 + scale) + shift
+
+    @staticmethod
+    def _modulate_jvp(norm_layer, x, tx, mod, tmod):
+        """LayerNorm + modulation of x and its tangent (one fused pass), written into the two halves of one buffer so
+        that the projections that follow map both in one GEMM without a copy."""
+        (shift, scale, _), (tshift, tscale, _) = mod, tmod
+        y, ty = ops.stacked_pair(x.shape, x.dtype, x.device)
+        flat = lambda m: m.reshape(-1, m.shape[-1])
+        ops.ln_modulate(x, flat(shift), flat(scale), tx, flat(tshift), flat(tscale), eps=norm_layer.eps, out=y, tout=ty)
+        return y, ty
+
+    @staticmethod
+    def _gated_residual_jvp(x, tx, res, tres, mod, tmod):
+        flat = lambda m: m.reshape(-1, m.shape[-1])
+        return ops.gated_residual(x, res, flat(mod[2]), tx, tres, flat(tmod[2]))
+
+    # ------------------------------------------------------------------ the reference's surface
+    def forward(
+        self,
+        x_B_T_H_W_D: torch.Tensor,
+        emb_B_T_D: torch.Tensor,
+        crossattn_emb: torch.Tensor,
+        rope_emb_L_1_1_D: Optional[torch.Tensor] = None,
+        adaln_lora_B_T_3D: Optional[torch.Tensor] = None,
+        extra_per_block_pos_emb: Optional[torch.Tensor] = None,
+    ) -> torch.Tensor:
+        x = x_B_T_H_W_D
+        if extra_per_block_pos_emb is not None:
+            x = x + extra_per_block_pos_emb
+        B, T, H, W, D = x.shape
+        shift, scale, gate = self._modulation(self.adaln_modulation_self_attn, emb_B_T_D, adaln_lora_B_T_3D, x)
+        n = self._modulate(self.layer_norm_self_attn, x, scale, shift)
+        r = self.self_attn(n.reshape(B, T * H * W, D), None, rope_emb=rope_emb_L_1_1_D).reshape(B, T, H, W, D)
+        x = x + gate * r
+        shift, scale, gate = self._modulation(self.adaln_modulation_cross_attn, emb_B_T_D, adaln_lora_B_T_3D, x)
+        n = self._modulate(self.layer_norm_cross_attn, x, scale, shift)
+        r = self.cross_attn(n.reshape(B, T * H * W, D), crossattn_emb, rope_emb=rope_emb_L_1_1_D).reshape(B, T, H, W, D)
+        x = r * gate + x
+        shift, scale, gate = self._modulation(self.adaln_modulation_mlp, emb_B_T_D, adaln_lora_B_T_3D, x)
+        n = self._modulate(self.layer_norm_mlp, x, scale, shift)
+        x = x + gate * self.mlp(n)
+        return x
+
+    # ------------------------------------------------------------------ forward mode
+    @torch.no_grad()
+    def forward_jvp(
+        self,
+        x_B_T_H_W_D: torch.Tensor,
+        tx_B_T_H_W_D: torch.Tensor,
+        emb_B_T_D: torch.Tensor,
+        temb_B_T_D: Optional[torch.Tensor],
+        crossattn_emb: torch.Tensor,
+        rope_emb_L_1_1_D: Optional[torch.Tensor] = None,
+        adaln_lora_B_T_3D: Optional[torch.Tensor] = None,
+        tadaln_lora_B_T_3D: Optional[torch.Tensor] = None,
+        extra_per_block_pos_emb: Optional[torch.Tensor] = None,
+    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """``(out, tout)``: the block's output and its derivative along ``(tx, temb, tadaln_lora)``; the text context
+        and the positional terms do not move."""
+        x, tx = x_B_T_H_W_D, tx_B_T_H_W_D
+        assert tx.shape == x.shape
+        if extra_per_block_pos_emb is not None:
+            x = x + extra_per_block_pos_emb
+        B, T, H, W, D = x.shape
+        flat = lambda z: z.reshape(B, T * H * W, D)
+        vid = lambda z: z.reshape(B, T, H, W, D)
+        args = (emb_B_T_D, temb_B_T_D, adaln_lora_B_T_3D, tadaln_lora_B_T_3D, x)
+
+        mod, tmod = self._modulation_jvp(self.adaln_modulation_self_attn, *args)
+        n, tn = self._modulate_jvp(self.layer_norm_self_attn, x, tx, mod, tmod)
+        r, tr = self.self_attn.forward_jvp(flat(n), flat(tn), rope_emb=rope_emb_L_1_1_D)
+        x, tx = self._gated_residual_jvp(x, tx, vid(r), vid(tr), mod, tmod)
+
+        mod, tmod = self._modulation_jvp(self.adaln_modulation_cross_attn, *args)
+        n, tn = self._modulate_jvp(self.layer_norm_cross_attn, x, tx, mod, tmod)
+        r, tr = self.cross_attn.forward_jvp(flat(n), flat(tn), crossattn_emb, None, rope_emb=rope_emb_L_1_1_D)
+        x, tx = self._gated_residual_jvp(x, tx, vid(r), vid(tr), mod, tmod)
+
+        mod, tmod = self._modulation_jvp(self.adaln_modulation_mlp, *args)
+        n, tn = self._modulate_jvp(self.layer_norm_mlp, x, tx, mod, tmod)
+        r, tr = self.mlp.forward_jvp(n, tn)
+        x, tx = self._gated_residual_jvp(x, tx, r, tr, mod, tmod)
+        return x, tx

@@ -100,6 +100,10 @@ def fwd_jvp(
     else:
         raise ValueError(f"out_layout={out_layout!r}")
     to = torch.empty_like(o) if have_tangent else None  # empty_like keeps o's strides
+    if have_tangent and out_layout == "blhd":
+        # o and to as the two halves of one buffer: a following linear layer maps both in one GEMM without a copy
+        both = torch.empty((2, B, Lq, H, d_v), device=q.device, dtype=q.dtype)
+        o, to = both[0].transpose(1, 2), both[1].transpose(1, 2)
     lse = torch.empty((B, H, Lq), device=q.device, dtype=torch.float32) if need_lse else None
 
     if key_lens is not None:
@@ -314,3 +318,122 @@ def norm_rope_bwd(
                                           torch.cuda.current_stream(x.device).cuda_stream)
     _lib.raise_for_status(status)
     return dx, dweight
+
+
+# ------------------------------------------------------------------ elementwise steps of the DiT block (+ tangents)
+def stacked_pair(shape, dtype, device):
+    """Two tensors of ``shape`` that are the halves of one ``[2, *shape]`` buffer (see :func:`as_stacked`)."""
+    both = torch.empty((2, *shape), device=device, dtype=dtype)
+    return both[0], both[1]
+
+
+def as_stacked(x: torch.Tensor, tx: torch.Tensor) -> Optional[torch.Tensor]:
+    """If ``x`` and ``tx`` are the two contiguous halves of one buffer, the ``[2 * x.shape[0], ...]`` view of it (no
+    copy); otherwise None."""
+    if (x.shape == tx.shape and x.dtype == tx.dtype and x.is_contiguous() and tx.is_contiguous() and x.dim() >= 1
+            and x._base is not None and x._base is tx._base
+            and tx.data_ptr() == x.data_ptr() + x.numel() * x.element_size()):
+        both = x._base
+        if both.is_contiguous() and both.data_ptr() == x.data_ptr() and both.numel() == 2 * x.numel():
+            return both.view(2 * x.shape[0], *x.shape[1:])
+    return None
+
+
+def _dense16(t: torch.Tensor) -> torch.Tensor:
+    return t if (t.is_contiguous() and t.data_ptr() % 16 == 0) else t.contiguous()
+
+
+def _check_elementwise(x: torch.Tensor) -> None:
+    if not x.is_cuda:
+        raise RuntimeError("cosmos attention (HIP) needs tensors on a GPU; there is no CPU path")
+    if x.dtype not in _DTYPES:
+        raise NotImplementedError(f"dtype={x.dtype} is not supported (bf16 / fp16)")
+
+
+def _launch(fn_name: str, desc, device) -> None:
+    lib = _lib.load_library()
+    with torch.cuda.device(device):
+        status = getattr(lib, fn_name)(ctypes.byref(desc), torch.cuda.current_stream(device).cuda_stream)
+    _lib.raise_for_status(status)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def ln_modulate(x, shift, scale, tx=None, tshift=None, tscale=None, eps: float = 1e-6, out=None, tout=None):
+    """``LayerNorm(x) * (1 + scale) + shift`` over the last dim (no affine parameters) and its tangent, one pass
+    (cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:1166-1167).  ``x``: ``[..., D]``; ``shift`` / ``scale``:
+    ``[G, D]`` with ``G`` dividing the number of rows (consecutive rows share a vector).  ``out`` / ``tout``: optional
+    preallocated outputs (e.g. the two halves of one stacked buffer).  Returns ``(y, ty)``."""
+    _check_elementwise(x)
+    D = x.shape[-1]
+    x = _dense16(x)
+    rows = x.numel() // D
+    shift, scale = _dense16(shift.to(x.dtype)).reshape(-1, D), _dense16(scale.to(x.dtype)).reshape(-1, D)
+    assert shift.shape == scale.shape and rows % shift.shape[0] == 0
+    if tx is not None:
+        assert tx.shape == x.shape and tx.dtype == x.dtype
+        tx = _dense16(tx)
+        tshift = None if tshift is None else _dense16(tshift.to(x.dtype)).reshape(-1, D)
+        tscale = None if tscale is None else _dense16(tscale.to(x.dtype)).reshape(-1, D)
+        assert (tshift is None or tshift.shape == shift.shape) and (tscale is None or tscale.shape == shift.shape)
+    y = torch.empty_like(x) if out is None else out
+    ty = (torch.empty_like(x) if tout is None else tout) if tx is not None else None
+    assert y.is_contiguous() and y.shape == x.shape and (ty is None or (ty.is_contiguous() and ty.shape == x.shape))
+    d = _lib.LnModulateDesc()
+    d.abi_version, d.dtype = _lib.ABI_VERSION, _DTYPES[x.dtype]
+    d.D, d.rows_per_group, d.eps, d.reserved, d.rows = D, rows // shift.shape[0], float(eps), 0, rows
+    d.x, d.tx, d.shift, d.scale = _ptr(x), _ptr(tx), _ptr(shift), _ptr(scale)
+    d.tshift, d.tscale = (_ptr(tshift), _ptr(tscale)) if tx is not None else (None, None)
+    d.y, d.ty = _ptr(y), _ptr(ty)
+    _launch("cosmos_ln_modulate", d, x.device)
+    return y, ty
+
+
+def gated_residual(x, res, gate, tx=None, tres=None, tgate=None, inplace: bool = False):
+    """``x + gate * res`` and its tangent ``tx + tgate * res + gate * tres`` in one pass
+    (cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:1199, :1231, :1241).  ``gate``: ``[G, D]`` as in
+    :func:`ln_modulate`.  ``inplace`` overwrites ``x`` / ``tx``.  Returns ``(out, tout)``."""
+    _check_elementwise(x)
+    D = x.shape[-1]
+    assert res.shape == x.shape and res.dtype == x.dtype
+    xs, res = _dense16(x), _dense16(res)
+    rows = xs.numel() // D
+    gate = _dense16(gate.to(x.dtype)).reshape(-1, D)
+    assert rows % gate.shape[0] == 0
+    if tx is not None:
+        assert tres is not None and tx.shape == x.shape and tres.shape == x.shape
+        txs, tres = _dense16(tx), _dense16(tres)
+        tgate = None if tgate is None else _dense16(tgate.to(x.dtype)).reshape(-1, D)
+    else:
+        txs = None
+    out = xs if (inplace and xs is x) else torch.empty_like(xs)
+    tout = None if tx is None else (txs if (inplace and txs is tx) else torch.empty_like(txs))
+    d = _lib.GatedResidualDesc()
+    d.abi_version, d.dtype = _lib.ABI_VERSION, _DTYPES[x.dtype]
+    d.D, d.rows_per_group, d.rows = D, rows // gate.shape[0], rows
+    d.x, d.tx, d.res, d.tres = _ptr(xs), _ptr(txs), _ptr(res), (_ptr(tres) if tx is not None else None)
+    d.gate, d.tgate = _ptr(gate), (_ptr(tgate) if tx is not None else None)
+    d.out, d.tout = _ptr(out), _ptr(tout)
+    _launch("cosmos_gated_residual", d, x.device)
+    return out, tout
+
+
+def gelu(h, th=None, inplace: bool = False):
+    """Exact (erf) GELU and its tangent ``th * gelu'(h)`` in one pass (``nn.GELU()`` of
+    cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:225).  Returns ``(a, ta)``."""
+    _check_elementwise(h)
+    hs = _dense16(h)
+    assert hs.numel() % 8 == 0, "the number of elements must be a multiple of 8"
+    ths = None
+    if th is not None:
+        assert th.shape == h.shape and th.dtype == h.dtype
+        ths = _dense16(th)
+    a = hs if (inplace and hs is h) else torch.empty_like(hs)
+    ta = None if th is None else (ths if (inplace and ths is th) else torch.empty_like(ths))
+    d = _lib.GeluDesc()
+    d.abi_version, d.dtype, d.n = _lib.ABI_VERSION, _DTYPES[h.dtype], hs.numel()
+    d.h, d.th, d.a, d.ta = _ptr(hs), _ptr(ths), _ptr(a), _ptr(ta)
+    _launch("cosmos_gelu", d, h.device)
+    return a, ta

@@ -194,6 +194,50 @@ COSMOS_ATTN_API size_t cosmos_norm_rope_bwd_workspace_bytes(const cosmos_norm_ro
 COSMOS_ATTN_API int cosmos_norm_rope_bwd(const cosmos_norm_rope_bwd_desc *desc, void *workspace, size_t workspace_bytes,
                                          void *stream);
 
+/*
+ * Elementwise steps of the DiT block with optional forward-mode tangents (networks/minimal_v4_dit.py:1119-1242), each one
+ * pass over 16-bit tensors with fp32 arithmetic.  Tensors are dense row-major [rows, D]; a modulation vector [groups, D]
+ * is shared by `rows_per_group` consecutive rows (the H*W tokens of one (batch, frame), :1150-1162).  Tangent pointers
+ * are optional: all NULL = values only.
+ *
+ * cosmos_ln_modulate:     y = LayerNorm(x) * (1 + scale) + shift           (:1166-1167; no affine parameters, eps :1031)
+ *                         ty = its derivative along (tx, tscale, tshift)    (tscale / tshift NULL = they do not move)
+ * cosmos_gated_residual:  out = x + gate * res                               (:1199, :1231, :1241)
+ *                         tout = tx + tgate * res + gate * tres              (out / tout may alias x / tx)
+ * cosmos_gelu:            a = gelu(h) (exact, erf form: nn.GELU() of :225),  ta = th * gelu'(h)
+ */
+typedef struct cosmos_ln_modulate_desc {
+    int32_t abi_version, dtype;
+    int32_t D, rows_per_group;     /* D % 8 == 0, D <= 8192; rows % rows_per_group == 0 */
+    float eps;
+    int32_t reserved;
+    int64_t rows;
+    const void *x, *tx;            /* [rows, D] */
+    const void *shift, *scale;     /* [rows / rows_per_group, D] */
+    const void *tshift, *tscale;   /* same shape, or NULL */
+    void *y, *ty;                  /* [rows, D] */
+} cosmos_ln_modulate_desc;
+
+typedef struct cosmos_gated_residual_desc {
+    int32_t abi_version, dtype;
+    int32_t D, rows_per_group;
+    int64_t rows;
+    const void *x, *tx, *res, *tres;   /* [rows, D]; tx, tres, tout NULL together */
+    const void *gate, *tgate;          /* [rows / rows_per_group, D]; tgate may be NULL */
+    void *out, *tout;
+} cosmos_gated_residual_desc;
+
+typedef struct cosmos_gelu_desc {
+    int32_t abi_version, dtype;
+    int64_t n;                         /* elements, n % 8 == 0 */
+    const void *h, *th;                /* th, ta NULL together */
+    void *a, *ta;
+} cosmos_gelu_desc;
+
+COSMOS_ATTN_API int cosmos_ln_modulate(const cosmos_ln_modulate_desc *desc, void *stream);
+COSMOS_ATTN_API int cosmos_gated_residual(const cosmos_gated_residual_desc *desc, void *stream);
+COSMOS_ATTN_API int cosmos_gelu(const cosmos_gelu_desc *desc, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -30,6 +30,11 @@ def dit_oracle():
 
 
 @pytest.fixture(scope="session")
+def block_oracle():
+    return entry.load_dit_block_oracle()
+
+
+@pytest.fixture(scope="session")
 def pkg():
     """The package with its HIP library loaded; fails loudly when the library is not built."""
     return entry.load_package()

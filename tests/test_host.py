@@ -15,7 +15,7 @@ HEADER = os.path.join(entry.REPO_ROOT, "include", "cosmos_attn_hip.h")
 
 def declared_symbols():
     text = open(HEADER).read()
-    return re.findall(r"COSMOS_ATTN_API\s+[\w\s\*]+?\b(cosmos_(?:attn|norm)_\w+)\s*\(", text)
+    return re.findall(r"COSMOS_ATTN_API\s+[\w\s\*]+?\b(cosmos_(?:attn|norm|ln|gated|gelu)\w*)\s*\(", text)
 
 
 def test_header_and_binding_agree(pkg):
@@ -248,6 +248,74 @@ def test_dit_attention_module_mirrors_reference_surface(pkg):
     with pytest.raises(RuntimeError, match="GPU"):          # no CPU path
         with torch.no_grad():
             m.bfloat16()(torch.zeros(1, 4, 64, dtype=torch.bfloat16))
+
+
+def test_block_elementwise_desc_layouts_and_status_codes(pkg):
+    L, lib = pkg._lib, pkg._lib.load_library()
+    assert ctypes.sizeof(L.LnModulateDesc) == 24 + 8 + 8 * 8 and L.LnModulateDesc.x.offset == 32
+    assert ctypes.sizeof(L.GatedResidualDesc) == 16 + 8 + 8 * 8 and L.GatedResidualDesc.x.offset == 24
+    assert ctypes.sizeof(L.GeluDesc) == 8 + 8 + 4 * 8 and L.GeluDesc.h.offset == 16
+    P = 0x7F0000000000   # never dereferenced: every case below is rejected on the host
+
+    def ln(**over):
+        D = L.LnModulateDesc()
+        D.abi_version, D.dtype, D.D, D.rows_per_group, D.eps, D.rows = L.ABI_VERSION, L.DTYPE_BF16, 256, 4, 1e-6, 16
+        D.x, D.shift, D.scale, D.y = P, P + 0x10000, P + 0x20000, P + 0x30000
+        for k, v in over.items():
+            setattr(D, k, v)
+        return D
+
+    for over, want in [(dict(abi_version=1), L.ST_BAD_ARG), (dict(rows=0), L.ST_BAD_ARG), (dict(scale=None), L.ST_BAD_ARG),
+                       (dict(tx=P + 0x40000), L.ST_BAD_ARG), (dict(tshift=P + 0x40000), L.ST_BAD_ARG), (dict(dtype=7), L.ST_UNSUPPORTED),
+                       (dict(D=8200), L.ST_UNSUPPORTED), (dict(D=252), L.ST_BAD_SHAPE), (dict(rows_per_group=5), L.ST_BAD_SHAPE),
+                       (dict(y=P + 0x30002), L.ST_BAD_STRIDE)]:
+        assert lib.cosmos_ln_modulate(ctypes.byref(ln(**over)), None) == want, over
+
+    def gr(**over):
+        D = L.GatedResidualDesc()
+        D.abi_version, D.dtype, D.D, D.rows_per_group, D.rows = L.ABI_VERSION, L.DTYPE_FP16, 64, 2, 8
+        D.x, D.res, D.gate, D.out = P, P + 0x10000, P + 0x20000, P
+        for k, v in over.items():
+            setattr(D, k, v)
+        return D
+
+    for over, want in [(dict(abi_version=0), L.ST_BAD_ARG), (dict(gate=None), L.ST_BAD_ARG), (dict(tx=P + 0x40000), L.ST_BAD_ARG),
+                       (dict(tgate=P + 0x40000), L.ST_BAD_ARG), (dict(dtype=3), L.ST_UNSUPPORTED), (dict(D=60), L.ST_BAD_SHAPE),
+                       (dict(rows=7), L.ST_BAD_SHAPE), (dict(res=P + 8), L.ST_BAD_STRIDE)]:
+        assert lib.cosmos_gated_residual(ctypes.byref(gr(**over)), None) == want, over
+
+    def ge(**over):
+        D = L.GeluDesc()
+        D.abi_version, D.dtype, D.n, D.h, D.a = L.ABI_VERSION, L.DTYPE_BF16, 64, P, P
+        for k, v in over.items():
+            setattr(D, k, v)
+        return D
+
+    for over, want in [(dict(abi_version=0), L.ST_BAD_ARG), (dict(n=0), L.ST_BAD_ARG), (dict(th=P + 0x100), L.ST_BAD_ARG),
+                       (dict(dtype=9), L.ST_UNSUPPORTED), (dict(n=12), L.ST_BAD_SHAPE), (dict(a=P + 4), L.ST_BAD_STRIDE)]:
+        assert lib.cosmos_gelu(ctypes.byref(ge(**over)), None) == want, over
+    with pytest.raises(RuntimeError, match="GPU"):       # no CPU path
+        pkg.gelu(torch.zeros(8, dtype=torch.bfloat16))
+
+
+def test_dit_block_mirrors_reference_surface(pkg):
+    m = pkg.Block(64, 48, 2, mlp_ratio=4.0, use_adaln_lora=True, adaln_lora_dim=8)
+    names = sorted(m.state_dict())
+    # parameter names of cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:1029-1082 (LayerNorms carry none)
+    assert names == sorted(
+        [f"{a}.{p}.weight" for a in ("self_attn", "cross_attn") for p in ("q_proj", "k_proj", "v_proj", "output_proj", "q_norm", "k_norm")]
+        + ["mlp.layer1.weight", "mlp.layer2.weight"]
+        + [f"adaln_modulation_{n}.{i}.weight" for n in ("self_attn", "cross_attn", "mlp") for i in (1, 2)])
+    assert m.mlp.layer1.weight.shape == (256, 64) and m.adaln_modulation_mlp[2].weight.shape == (192, 8)
+    assert m.cross_attn.k_proj.weight.shape == (64, 48) and m.self_attn.is_selfattn and not m.cross_attn.is_selfattn
+    m.init_weights()
+    assert float(m.adaln_modulation_mlp[2].weight.abs().max()) == 0.0       # the block starts as the identity
+    plain = pkg.Block(64, 48, 2)
+    assert sorted(k for k in plain.state_dict() if k.startswith("adaln")) == [f"adaln_modulation_{n}.1.weight" for n in ("cross_attn", "mlp", "self_attn")]
+    for name in ("forward", "forward_jvp", "init_weights", "reset_parameters", "set_context_parallel_group"):
+        assert callable(getattr(m, name))
+    with pytest.raises(NotImplementedError):
+        pkg.Block(64, 48, 2, image_context_dim=32)
 
 
 def test_status_to_exception_mapping(pkg):
