@@ -189,3 +189,61 @@ class Attention(nn.Module):
         out, tout = self._apply_stacked(self.output_proj, self._stack(o, to), True)
         shape = (*x.shape[:-1], out.shape[-1])
         return out.reshape(shape), tout.reshape(shape)
+
+
+class I2VCrossAttention(Attention):
+    """Cross-attention over a text context and an image context with separate key / value projections, the two results
+    summed before the output projection (cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:451-493).  ``context``
+    is the pair ``(text_context, img_context)``; parameter names as in the reference (``k_img``, ``v_img``,
+    ``k_img_norm``)."""
+
+    def __init__(self, *args, img_latent_dim: int = 1024, **kwargs):
+        super().__init__(*args, **kwargs)
+        inner_dim = self.head_dim * self.n_heads
+        self.k_img = nn.Linear(img_latent_dim, inner_dim, bias=False)
+        self.v_img = nn.Linear(img_latent_dim, inner_dim, bias=False)
+        self.k_img_norm = HeadRMSNormWeight(self.head_dim, eps=1e-6)
+
+    def init_weights(self) -> None:
+        super().init_weights()
+        torch.nn.init.trunc_normal_(self.k_img.weight, std=1.0 / math.sqrt(self._inner_dim))
+        torch.nn.init.trunc_normal_(self.v_img.weight, std=1.0 / math.sqrt(self._inner_dim))
+        self.k_img_norm.reset_parameters()
+
+    def compute_qkv(self, x, context, rope_emb=None):
+        text_context, img_context = context
+        q, k, v = super().compute_qkv(x, text_context, rope_emb)
+        k_img, _ = self._norm_rope(self._heads(self.k_img(img_context)), self.k_img_norm, None)
+        v_img = self._heads(self.v_img(img_context))
+        return q, k, v, k_img, v_img
+
+    def compute_attention(self, q, k, v, k_img, v_img):
+        result = self.attn_op(q, k, v)
+        result_img = self.attn_op(q, k_img, v_img)
+        return self.output_dropout(self.output_proj(result + result_img))
+
+    def forward(self, x, context=None, rope_emb=None, video_size=None):
+        del video_size
+        q, k, v, k_img, v_img = self.compute_qkv(x, context, rope_emb)
+        out = self.compute_attention(q, k, v, k_img, v_img)
+        return out.reshape(*x.shape[:-1], out.shape[-1])
+
+    @torch.no_grad()
+    def forward_jvp(self, x, tx, context=None, tcontext=None, rope_emb=None):
+        """``(out, tout)`` along ``tx``; the text and image contexts do not move."""
+        assert tcontext is None, "a moving context is not supported by the image-conditioned cross-attention"
+        assert tx is not None and tx.shape == x.shape
+        text_context, img_context = context
+        h = self._heads
+        q, tq = self._apply_stacked(self.q_proj, self._stack(x, tx), True)
+        q, tq = self._norm_rope(h(q), self.q_norm, rope_emb, h(tq))
+        k, _ = self._norm_rope(h(self.k_proj(text_context)), self.k_norm, rope_emb)
+        k_img, _ = self._norm_rope(h(self.k_img(img_context)), self.k_img_norm, None)
+        v, v_img = h(self.v_proj(text_context)), h(self.v_img(img_context))
+        o, to = self.attn_op.forward_jvp(q, k, v, tq)
+        o2, to2 = self.attn_op.forward_jvp(q, k_img, v_img, tq)
+        o.add_(o2)
+        to.add_(to2)
+        out, tout = self._apply_stacked(self.output_proj, self._stack(o, to), True)
+        shape = (*x.shape[:-1], out.shape[-1])
+        return out.reshape(shape), tout.reshape(shape)

@@ -23,7 +23,7 @@ import torch
 from torch import nn
 
 from . import ops
-from .dit_attention import Attention
+from .dit_attention import Attention, I2VCrossAttention
 
 
 class GPT2FeedForward(nn.Module):
@@ -73,15 +73,17 @@ class Block(nn.Module):
         use_wan_fp32_strategy: bool = False,
     ):
         super().__init__()
-        if image_context_dim is not None:
-            raise NotImplementedError("the image-conditioned cross-attention (I2VCrossAttention) is not built")
         if use_wan_fp32_strategy:
             raise NotImplementedError("use_wan_fp32_strategy is not built")
         self.x_dim = x_dim
         self.layer_norm_self_attn = nn.LayerNorm(x_dim, elementwise_affine=False, eps=1e-6)
         self.self_attn = Attention(x_dim, None, num_heads, x_dim // num_heads, qkv_format="bshd", backend=backend)
         self.layer_norm_cross_attn = nn.LayerNorm(x_dim, elementwise_affine=False, eps=1e-6)
-        self.cross_attn = Attention(x_dim, context_dim, num_heads, x_dim // num_heads, qkv_format="bshd", backend=backend)
+        if image_context_dim is None:
+            self.cross_attn = Attention(x_dim, context_dim, num_heads, x_dim // num_heads, qkv_format="bshd", backend=backend)
+        else:   # crossattn_emb is then the pair (text context, image context)
+            self.cross_attn = I2VCrossAttention(x_dim, context_dim, num_heads, x_dim // num_heads,
+                                                img_latent_dim=image_context_dim, qkv_format="bshd", backend=backend)
         self.layer_norm_mlp = nn.LayerNorm(x_dim, elementwise_affine=False, eps=1e-6)
         self.mlp = GPT2FeedForward(x_dim, int(x_dim * mlp_ratio))
 

@@ -26,7 +26,10 @@ from typing import Dict, Optional
 
 def block_torch(weights: Dict[str, "torch.Tensor"], x, emb, crossattn_emb, rope_angles=None, num_heads: int = 8,
                 adaln_lora=None, tx=None, temb=None, tadaln_lora=None, dtype=None, keep_graph_input=None):
-    """weights: the block's state dict.  x: [B, T, H, W, D]; emb: [B, T, D]; crossattn_emb: [B, Mk, Kc];
+    """weights: the block's state dict.  x: [B, T, H, W, D]; emb: [B, T, D]; crossattn_emb: [B, Mk, Kc], or the pair
+    (text context, image context [B, Mi, Ki]) when the state dict holds the image-conditioned cross-attention
+    (``cross_attn.k_img.weight`` ...: minimal_v4_dit.py:451-493, the two attention results are summed before the output
+    projection);
     rope_angles: [T*H*W, D/num_heads] or None; adaln_lora: [B, T, 3 D] (required iff the state dict holds the
     LoRA form of the modulation).  Returns (out, tout); tout is None without tx."""
     import torch
@@ -36,6 +39,10 @@ def block_torch(weights: Dict[str, "torch.Tensor"], x, emb, crossattn_emb, rope_
     dt = dtype or torch.float32
     f = lambda t: None if t is None else torch.as_tensor(t).detach().to("cpu", dt)
     w = {k: f(v) for k, v in weights.items()}
+    img_ctx = None
+    if isinstance(crossattn_emb, (tuple, list)):
+        crossattn_emb, img_ctx = crossattn_emb
+        img_ctx = f(img_ctx)
     x, emb, ctx, lora, tx, temb, tlora = (f(t) for t in (x, emb, crossattn_emb, adaln_lora, tx, temb, tadaln_lora))
     if keep_graph_input is not None:
         x = keep_graph_input.to(dt)
@@ -56,14 +63,18 @@ def block_torch(weights: Dict[str, "torch.Tensor"], x, emb, crossattn_emb, rope_
             return n
         return n * torch.cos(rope) + torch.cat([-n[..., hd // 2:], n[..., : hd // 2]], dim=-1) * torch.sin(rope)
 
-    def attention(prefix, xq, c, rope):
+    def attention(prefix, xq, c, rope, c_img=None):
         heads = lambda t: t.reshape(t.shape[0], -1, num_heads, hd)
+        sdpa = lambda q_, k_, v_: F.scaled_dot_product_attention(q_.transpose(1, 2), k_.transpose(1, 2), v_.transpose(1, 2)).transpose(1, 2)
         q = norm_rope(heads(F.linear(xq, w[prefix + "q_proj.weight"])), w[prefix + "q_norm.weight"], rope)
         k = norm_rope(heads(F.linear(c, w[prefix + "k_proj.weight"])), w[prefix + "k_norm.weight"], rope)
         v = heads(F.linear(c, w[prefix + "v_proj.weight"]))
         with sdpa_kernel([SDPBackend.MATH]):
-            o = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))
-        return F.linear(o.transpose(1, 2).flatten(-2), w[prefix + "output_proj.weight"])
+            o = sdpa(q, k, v)
+            if c_img is not None:
+                k_img = norm_rope(heads(F.linear(c_img, w[prefix + "k_img.weight"])), w[prefix + "k_img_norm.weight"], None)
+                o = o + sdpa(q, k_img, heads(F.linear(c_img, w[prefix + "v_img.weight"])))
+        return F.linear(o.flatten(-2), w[prefix + "output_proj.weight"])
 
     def fwd(x_, e_, l_):
         ln = lambda t: F.layer_norm(t, (D,), eps=1e-6)
@@ -72,7 +83,7 @@ def block_torch(weights: Dict[str, "torch.Tensor"], x, emb, crossattn_emb, rope_
         x_ = x_ + gate * attention("self_attn.", n, n, a).reshape(B, T, H, W, D)
         shift, scale, gate = modulation("cross_attn", e_, l_)
         n = (ln(x_) * (1 + scale) + shift).reshape(B, T * H * W, D)
-        x_ = attention("cross_attn.", n, ctx, None).reshape(B, T, H, W, D) * gate + x_
+        x_ = attention("cross_attn.", n, ctx, None, img_ctx).reshape(B, T, H, W, D) * gate + x_
         shift, scale, gate = modulation("mlp", e_, l_)
         n = ln(x_) * (1 + scale) + shift
         return x_ + gate * F.linear(F.gelu(F.linear(n, w["mlp.layer1.weight"])), w["mlp.layer2.weight"])

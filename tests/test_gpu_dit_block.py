@@ -75,6 +75,36 @@ def test_block_2b_widths_reduced_length(pkg, oracle, nr_oracle, block_oracle, gp
     run(pkg, oracle, nr_oracle, block_oracle, gpu, B=1, T=3, Hh=8, W=16, D=2048, H=16, Mk=512, Kc=1024, lora_dim=256, seed=3)
 
 
+def test_block_with_image_context(pkg, oracle, nr_oracle, block_oracle, gpu):
+    """image_context_dim: the cross-attention also attends to an image context (minimal_v4_dit.py:451-493)."""
+    B, T, Hh, W, D, H, Mk, Kc, Mi, Ki = 2, 2, 4, 6, 256, 2, 20, 96, 12, 80
+    torch.manual_seed(7)
+    m = pkg.Block(D, Kc, H, use_adaln_lora=True, adaln_lora_dim=16, image_context_dim=Ki)
+    m.init_weights()
+    with torch.no_grad():
+        for mod in (m.adaln_modulation_self_attn, m.adaln_modulation_cross_attn, m.adaln_modulation_mlp):
+            mod[-1].weight.copy_(torch.randn_like(mod[-1].weight) / 4.0)
+    m = m.to(device=gpu, dtype=torch.bfloat16).eval()
+    assert "cross_attn.k_img.weight" in m.state_dict() and "cross_attn.k_img_norm.weight" in m.state_dict()
+    g = torch.Generator().manual_seed(8)
+    r = lambda *s: torch.randn(*s, generator=g)
+    x, tx = r(B, T, Hh, W, D).bfloat16(), (0.3 * r(B, T, Hh, W, D)).bfloat16()
+    emb, temb, lora = r(B, T, D).bfloat16(), (0.3 * r(B, T, D)).bfloat16(), (0.3 * r(B, T, 3 * D)).bfloat16()
+    ctx, img = r(B, Mk, Kc).bfloat16(), r(B, Mi, Ki).bfloat16()
+    hd = D // H
+    angles = torch.from_numpy(nr_oracle.rope_angles_3d(T, Hh, W, hd))
+    rope = angles.reshape(-1, 1, 1, hd).to(gpu)
+    d = lambda t: t.to(gpu)
+    with torch.no_grad():
+        out = m(d(x), d(emb), (d(ctx), d(img)), rope, d(lora))
+    out2, tout = m.forward_jvp(d(x), d(tx), d(emb), d(temb), (d(ctx), d(img)), rope, d(lora), None)
+    want, twant = block_oracle.block_torch(m.state_dict(), x, emb, (ctx, img), angles.numpy(), H, lora, tx, temb, None)
+    check(oracle, "out", out, want)
+    check(oracle, "out (jvp call)", out2, want)
+    check(oracle, "tout", tout, twant)
+    check(oracle, "out - x", out.float().cpu() - x.float(), want - x.float(), rel_l2=2e-2)
+
+
 def test_fresh_block_is_the_identity(pkg, nr_oracle, gpu):
     """minimal_v4_dit.py:1095-1111: after init_weights the gates are zero."""
     torch.manual_seed(0)

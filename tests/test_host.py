@@ -314,8 +314,11 @@ def test_dit_block_mirrors_reference_surface(pkg):
     assert sorted(k for k in plain.state_dict() if k.startswith("adaln")) == [f"adaln_modulation_{n}.1.weight" for n in ("cross_attn", "mlp", "self_attn")]
     for name in ("forward", "forward_jvp", "init_weights", "reset_parameters", "set_context_parallel_group"):
         assert callable(getattr(m, name))
+    i2v = pkg.Block(64, 48, 2, image_context_dim=32)
+    assert isinstance(i2v.cross_attn, pkg.I2VCrossAttention) and i2v.cross_attn.k_img.weight.shape == (64, 32)
+    assert {"cross_attn.k_img.weight", "cross_attn.v_img.weight", "cross_attn.k_img_norm.weight"} <= set(i2v.state_dict())
     with pytest.raises(NotImplementedError):
-        pkg.Block(64, 48, 2, image_context_dim=32)
+        pkg.Block(64, 48, 2, use_wan_fp32_strategy=True)
 
 
 def test_status_to_exception_mapping(pkg):

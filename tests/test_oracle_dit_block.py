@@ -146,3 +146,32 @@ def test_elementwise_oracles_match_closed_forms(block_oracle):
     o, to = block_oracle.gated_residual_torch(xx, res, gate, txx, tres, tgate, rows_per_group=rpg)
     np.testing.assert_allclose(o.numpy(), xx.numpy() + rep(gate) * res.numpy(), atol=2e-6)
     np.testing.assert_allclose(to.numpy(), txx.numpy() + rep(tgate) * res.numpy() + rep(gate) * tres.numpy(), atol=2e-6)
+
+
+def test_image_branch_is_a_second_attention_summed_before_the_output_projection(block_oracle, dit_oracle):
+    """minimal_v4_dit.py:480-483: out_proj(attn(q, k, v) + attn(q, k_img, v_img)).  With zero gates on the other two
+    sub-layers the block reduces to x + gate * that, which is rebuilt here from the pinned attention-module oracle by
+    linearity of the output projection."""
+    B, T, Hh, W, D, H, Mk, Kc, Mi, Ki = 1, 1, 2, 3, 32, 2, 5, 24, 4, 20
+    w = make_block_weights(D, Kc, H, 0, 51)
+    g = torch.Generator().manual_seed(52)
+    r = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    w["cross_attn.k_img.weight"], w["cross_attn.v_img.weight"] = r(D, Ki) / Ki ** 0.5, r(D, Ki) / Ki ** 0.5
+    w["cross_attn.k_img_norm.weight"] = 1 + 0.2 * r(D // H)
+    for name in ("self_attn", "mlp"):                       # gates of the other sub-layers to zero
+        w[f"adaln_modulation_{name}.1.weight"][2 * D:] = 0
+    i = inputs(B, T, Hh, W, D, Mk, Kc, False, 53)
+    img = r(B, Mi, Ki)
+    out, _ = block_oracle.block_torch(w, i["x"], i["emb"], (i["ctx"], img), None, H, dtype=torch.float64)
+
+    m = torch.nn.functional.silu(i["emb"]) @ w["adaln_modulation_cross_attn.1.weight"].T
+    shift, scale, gate = (c[:, :, None, None, :] for c in m.chunk(3, dim=-1))
+    n = (torch.nn.functional.layer_norm(i["x"], (D,), eps=1e-6) * (1 + scale) + shift).reshape(B, -1, D)
+    text = {k[len("cross_attn."):]: v for k, v in w.items() if k.startswith("cross_attn.") and "img" not in k}
+    image = dict(text)
+    image["k_proj.weight"], image["v_proj.weight"], image["k_norm.weight"] = (w["cross_attn.k_img.weight"], w["cross_attn.v_img.weight"],
+                                                                              w["cross_attn.k_img_norm.weight"])
+    a1, _ = dit_oracle.attention_module_torch(text, n, i["ctx"], None, H, D // H, dtype=torch.float64)
+    a2, _ = dit_oracle.attention_module_torch(image, n, img, None, H, D // H, dtype=torch.float64)
+    want = i["x"] + gate * (a1 + a2).reshape(i["x"].shape)
+    np.testing.assert_allclose(out.numpy(), want.numpy(), atol=1e-10)
