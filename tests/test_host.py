@@ -321,6 +321,40 @@ def test_dit_block_mirrors_reference_surface(pkg):
         pkg.Block(64, 48, 2, use_wan_fp32_strategy=True)
 
 
+def test_rope_position_table_mirrors_reference(pkg, nr_oracle):
+    """VideoRopePosition3DEmb (cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:534-661): layout, fps and NTK rules."""
+    import numpy as np
+
+    T, H, W, D = 3, 4, 5, 128
+    pe = pkg.VideoRopePosition3DEmb(head_dim=D, len_h=8, len_w=8, len_t=8)
+    assert sorted(pe.state_dict()) == ["dim_spatial_range", "dim_temporal_range", "seq"] and pe.seq_dim == 0
+    x = torch.zeros(1, T, H, W, 16)
+    e = pe(x, fps=torch.tensor([24.0]))
+    assert e.shape == (T * H * W, 1, 1, D) and e.dtype == torch.float32
+    # at the base frame rate the table is the plain 3-D one (the oracle's construction, pinned on its own)
+    np.testing.assert_allclose(e.reshape(-1, D).numpy(), nr_oracle.rope_angles_3d(T, H, W, D), rtol=1e-6, atol=1e-6)
+    # half the frame rate: the temporal angles double (frame index / fps * base_fps), the spatial ones stay
+    e12 = pe(x, fps=torch.tensor([12.0])).reshape(T, H, W, D)
+    e24 = e.reshape(T, H, W, D)
+    dim_h = D // 6 * 2
+    dim_t = D - 2 * dim_h
+    assert torch.allclose(e12[..., : dim_t // 2], 2 * e24[..., : dim_t // 2]) and torch.equal(e12[..., dim_t // 2: D // 2], e24[..., dim_t // 2: D // 2])
+    # image batch: no fps, one frame
+    assert pe(torch.zeros(2, 1, H, W, 16)).shape == (H * W, 1, 1, D)
+    with pytest.raises(AssertionError, match="T should be 1"):
+        pe(x)
+    with pytest.raises(AssertionError, match="exceed the maximum"):
+        pe(torch.zeros(1, 1, 9, 2, 16))
+    # NTK extrapolation: ratio r stretches the base to 10000 * r ** (dim / (dim - 2)) on that axis only
+    pe2 = pkg.VideoRopePosition3DEmb(head_dim=D, len_h=8, len_w=8, len_t=8, h_extrapolation_ratio=2.0, enable_fps_modulation=False)
+    e2 = pe2(x).reshape(T, H, W, D)
+    j = 3                                   # some channel of the h block
+    want = 2.0 / (10000.0 * 2.0 ** (dim_h / (dim_h - 2))) ** (2 * j / dim_h)     # position h = 2
+    assert abs(float(e2[0, 2, 0, dim_t // 2 + j]) - want) < 1e-6 * want + 1e-9
+    assert torch.equal(e2[..., dim_t // 2 + dim_h // 2: D // 2], e24[..., dim_t // 2 + dim_h // 2: D // 2])   # w block untouched
+    assert torch.allclose(e2[..., : dim_t // 2], e24[..., : dim_t // 2])            # fps modulation off = base frame rate
+
+
 def test_status_to_exception_mapping(pkg):
     L = pkg._lib
     L.raise_for_status(L.ST_OK)
