@@ -135,6 +135,11 @@ struct AttnParams {
     const int32_t* key_lens;   // nullable
     int H, Lq, Lkv, n_tiles, causal;
     float sm_scale, scale_log2;
+    // forward-only kernel: workgroups [0, n_full) each own a (query block, head) pair; the remaining pairs are cut into
+    // `splits` key ranges, one workgroup each, which leave unnormalised partial results for attn_combine_kernel
+    int n_qt, n_full, n_rem, splits;
+    float* part_acc;           // [(pair - n_full) * splits + split][kSymBlockM][d_v]
+    float2* part_ml;           // same leading index, [kSymBlockM]: (running max in log2 units, row sum)
 };
 
 extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -707,7 +712,12 @@ attn_fwd_sym_kernel(const AttnParams p) {
     constexpr int IN_FLIGHT = C::GROUP_LOADS;
     constexpr int WAIT_FILLS = (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14) | 0x0F70;
 
-    const int qt = blockIdx.x, bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
+    // 1-D grid: block id -> (pair, key range); pair = query block + n_qt * (batch * H + head)
+    const int bid = blockIdx.x;
+    const bool partial = bid >= p.n_full && p.splits > 1;
+    const int pair = partial ? p.n_full + (bid - p.n_full) / p.splits : bid;
+    const int split = partial ? (bid - p.n_full) % p.splits : 0;
+    const int qt = pair % p.n_qt, bh = pair / p.n_qt, b = bh / p.H, h = bh % p.H;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 31, hh = lane >> 5;
@@ -718,7 +728,10 @@ attn_fwd_sym_kernel(const AttnParams p) {
     if (p.key_lens) { const int kl = p.key_lens[b]; kv_len = kl < kv_len ? (kl < 0 ? 0 : kl) : kv_len; }
     int n_tiles = (kv_len + kBlockN - 1) / kBlockN;
     if (p.causal) { const int lim = (qt * kSymBlockM + kSymBlockM + kBlockN - 1) / kBlockN; n_tiles = n_tiles < lim ? n_tiles : lim; }
-    const int n_steps = (n_tiles + 1) / 2;   // (a last step tile that sticks out past n_tiles is masked like any tail)
+    const int n_steps_all = (n_tiles + 1) / 2;   // (a last step tile that sticks out past n_tiles is masked like any tail)
+    // this workgroup's share of the sweep: positions [u_lo, u_lo + n_steps)
+    const int u_lo = partial ? (int)((int64_t)split * n_steps_all / p.splits) : 0;
+    const int n_steps = partial ? (int)((int64_t)(split + 1) * n_steps_all / p.splits) - u_lo : n_steps_all;
 
     char* const kring = smem + C::KRING_OFF;
     char* const vring = smem + C::VRING_OFF;
@@ -726,10 +739,9 @@ attn_fwd_sym_kernel(const AttnParams p) {
     const __amdgpu_buffer_rsrc_t kv_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<char*>(p.kv) + (size_t)bh * p.n_tiles * TILE_BYTES, 0, p.n_tiles * TILE_BYTES, 0x00020000);
     // sweep order (in step tiles): see attn_fwd_jvp_kernel
-    const int n_sweep = n_steps > 0 ? n_steps : 1;
-    const int wg_linear = blockIdx.x + gridDim.x * blockIdx.y;
-    const int shift = p.causal ? 0 : (((wg_linear >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
-    auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane((u + shift) % n_sweep); };
+    const int n_sweep = n_steps_all > 0 ? n_steps_all : 1;
+    const int shift = p.causal ? 0 : (((pair >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
+    auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane((u_lo + u + shift) % n_sweep); };
     auto wrap_inc = [&](int t) { ++t; return t >= n_sweep ? t - n_sweep : t; };
     // this wavefront's run of fragments inside a K slot / V slot (never crosses a packed tile)
     const int kf0 = (wave * C::K_LOADS) % (2 * C::K_FR), vf0 = (wave * C::V_LOADS) % (2 * C::VT_FR);
@@ -802,6 +814,24 @@ attn_fwd_sym_kernel(const AttnParams p) {
 
     // ---- epilogue: O = acc / l ; LSE = (m + log2 l) ln 2 ----
     const float l_tot = w.l_run + __shfl_xor(w.l_run, 32);
+    if (partial) {
+        // a key range only: leave acc, m, l as they are for attn_combine_kernel (rows past Lq are written too and
+        // never combined)
+        const int64_t slot = (int64_t)(pair - p.n_full) * p.splits + split;
+        const int wrow = wave * 32 + j;
+        float* pa = p.part_acc + (slot * kSymBlockM + wrow) * DV;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = 32 * db + 8 * g + 4 * hh;
+                if (d < DV)
+                    *reinterpret_cast<float4*>(pa + d) = make_float4(w.acc[db][4 * g], w.acc[db][4 * g + 1], w.acc[db][4 * g + 2], w.acc[db][4 * g + 3]);
+            }
+        }
+        if (hh == 0) p.part_ml[slot * kSymBlockM + wrow] = make_float2(w.m_run, l_tot);
+        return;
+    }
     const float inv_l = 1.0f / l_tot;
     if (row < p.Lq) {
         T* op = reinterpret_cast<T*>(p.o) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)row * p.o_sl;
@@ -820,6 +850,38 @@ attn_fwd_sym_kernel(const AttnParams p) {
         }
         if (p.lse && hh == 0) p.lse[(int64_t)bh * p.Lq + row] = (w.m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
     }
+}
+
+// Merge the key-range partial results of one query row:  M = max m_i,  w_i = 2^(m_i - M),  L = sum l_i w_i,
+// O = sum acc_i w_i / L,  LSE = (M + log2 L) ln 2.  One thread per (row, 4 output channels); fixed order over the ranges.
+template <typename T>
+__global__ void __launch_bounds__(256) attn_combine_kernel(const AttnParams p, int dv) {
+    typedef typename VecOf<T>::v4 V4;
+    const int tpr = dv / 4;                                   // threads per row
+    const int64_t r = (int64_t)blockIdx.x * (256 / tpr) + threadIdx.x / tpr;   // row among the split pairs' rows
+    const int c = (threadIdx.x % tpr) * 4;
+    const int pair_i = (int)(r / kSymBlockM), wrow = (int)(r % kSymBlockM);
+    const int pair = p.n_full + pair_i;
+    const int qt = pair % p.n_qt, bh = pair / p.n_qt, b = bh / p.H, h = bh % p.H;
+    const int row = qt * kSymBlockM + wrow;
+    if (pair_i >= p.n_rem || row >= p.Lq) return;
+    const int64_t slot0 = (int64_t)pair_i * p.splits;
+    float M = -INFINITY;
+    for (int i = 0; i < p.splits; ++i) M = fmaxf(M, p.part_ml[(slot0 + i) * kSymBlockM + wrow].x);
+    float L = 0.f, o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+    for (int i = 0; i < p.splits; ++i) {
+        const float2 ml = p.part_ml[(slot0 + i) * kSymBlockM + wrow];
+        const float wgt = __builtin_amdgcn_exp2f(ml.x - M);
+        const float4 a = *reinterpret_cast<const float4*>(p.part_acc + ((slot0 + i) * kSymBlockM + wrow) * dv + c);
+        L += ml.y * wgt;
+        o0 += a.x * wgt; o1 += a.y * wgt; o2 += a.z * wgt; o3 += a.w * wgt;
+    }
+    const float inv_l = 1.0f / L;
+    T* op = reinterpret_cast<T*>(p.o) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)row * p.o_sl;
+    V4 ov;
+    ov[0] = (T)(o0 * inv_l); ov[1] = (T)(o1 * inv_l); ov[2] = (T)(o2 * inv_l); ov[3] = (T)(o3 * inv_l);
+    *reinterpret_cast<V4*>(op + c) = ov;
+    if (p.lse && c == 0) p.lse[(int64_t)bh * p.Lq + row] = (M + __builtin_log2f(L)) * 0.6931471805599453f;
 }
 
 // ------------------------------------------------------------------------------------------------ host
@@ -882,6 +944,39 @@ int n_tiles_of(const cosmos_attn_desc* d) { return (d->Lkv + kBlockN - 1) / kBlo
 // workspace = packed tiles [B*H][n_tiles][tile bytes]
 size_t tiles_bytes_of(const cosmos_attn_desc* d) { return (size_t)d->B * d->H * n_tiles_of(d) * tile_bytes_of(d); }
 
+// Forward only: how the (query block, head) pairs are dealt out.  One workgroup fits on a compute unit, so a launch
+// runs in rounds of kNumCUs workgroups; when the last round is less than half full its pairs are cut along the keys
+// into as many ranges as fill it, and a small second kernel merges the ranges.
+constexpr int kNumCUs = 256;
+constexpr int kMaxSplits = 16;
+constexpr int kMinStepsPerSplit = 4;
+struct SplitPlan { int n_qt, n_pairs, n_full, n_rem, splits; };
+SplitPlan plan_split(const cosmos_attn_desc* d) {
+    SplitPlan s;
+    s.n_qt = (d->Lq + kSymBlockM - 1) / kSymBlockM;
+    s.n_pairs = s.n_qt * d->B * d->H;
+    s.n_rem = 0; s.splits = 1; s.n_full = s.n_pairs;
+    if (d->causal || d->key_lens) return s;          // key ranges of equal work only
+    const int rem = s.n_pairs % kNumCUs;
+    const int n_steps = (n_tiles_of(d) + 1) / 2;
+    if (rem == 0 || rem > kNumCUs / 2) return s;
+    int splits = kNumCUs / rem;
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    if (splits > n_steps / kMinStepsPerSplit) splits = n_steps / kMinStepsPerSplit;
+    if (splits < 2) return s;
+    s.n_rem = rem; s.n_full = s.n_pairs - rem; s.splits = splits;
+    return s;
+}
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+// partial results of the split pairs: fp32 accumulators [slots][kSymBlockM][d_v], then (max, sum) [slots][kSymBlockM]
+size_t partial_bytes_of(const cosmos_attn_desc* d) {
+    if (mode_of(d) != MODE_FWD) return 0;
+    const SplitPlan s = plan_split(d);
+    if (s.splits < 2) return 0;
+    const size_t slots = (size_t)s.n_rem * s.splits;
+    return align256(slots * kSymBlockM * d->d_v * sizeof(float)) + align256(slots * kSymBlockM * sizeof(float2));
+}
+
 int validate(const cosmos_attn_desc* d) {
     if (!d) return COSMOS_ATTN_BAD_ARG;
     if (d->abi_version != COSMOS_ATTN_ABI_VERSION) return COSMOS_ATTN_BAD_ARG;
@@ -928,7 +1023,7 @@ COSMOS_ATTN_API const char* cosmos_attn_status_string(int status) {
 
 COSMOS_ATTN_API size_t cosmos_attn_workspace_bytes(const cosmos_attn_desc* d) {
     if (validate(d) != COSMOS_ATTN_OK) return 0;
-    return tiles_bytes_of(d);
+    return align256(tiles_bytes_of(d)) + partial_bytes_of(d);
 }
 
 COSMOS_ATTN_API int cosmos_attn_pack_kv(const cosmos_attn_desc* d, void* workspace, size_t workspace_bytes, void* stream) {
@@ -947,7 +1042,12 @@ COSMOS_ATTN_API int cosmos_attn_pack_kv(const cosmos_attn_desc* d, void* workspa
     return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
 }
 
-COSMOS_ATTN_API int cosmos_attn_run(const cosmos_attn_desc* d, const void* workspace, size_t workspace_bytes, void* stream) {
+}  // extern "C"
+
+namespace {
+// `scratch`: where key-range partial results may go (null: never split).  cosmos_attn_run only reads its workspace, so
+// that several runs may share one re-tiled K/V image; the one-call entry point owns the workspace and passes its tail.
+int run_impl(const cosmos_attn_desc* d, const void* workspace, size_t workspace_bytes, void* scratch, void* stream) {
     const int st = validate(d);
     if (st != COSMOS_ATTN_OK) return st;
     if (!workspace || workspace_bytes < cosmos_attn_workspace_bytes(d) || !aligned16(workspace)) return COSMOS_ATTN_WORKSPACE_TOO_SMALL;
@@ -967,16 +1067,48 @@ COSMOS_ATTN_API int cosmos_attn_run(const cosmos_attn_desc* d, const void* works
     ap.sm_scale = d->sm_scale; ap.scale_log2 = d->sm_scale * 1.4426950408889634f;
     const size_t lds = lds_bytes_of(d);
     if (!allow_lds((const void*)fn, lds)) return COSMOS_ATTN_LAUNCH_FAILED;
-    const int block_m = mode == MODE_FWD ? kSymBlockM : kBlockM;
-    const int n_qt = (d->Lq + block_m - 1) / block_m;
-    hipLaunchKernelGGL(fn, dim3(n_qt, d->B * d->H), dim3(mode == MODE_FWD ? 64 * kSymWaves : kAttnThreads), lds, (hipStream_t)stream, ap);
-    return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
+    ap.n_qt = 0; ap.n_full = 0; ap.n_rem = 0; ap.splits = 1; ap.part_acc = nullptr; ap.part_ml = nullptr;
+    if (mode != MODE_FWD) {
+        const int n_qt = (d->Lq + kBlockM - 1) / kBlockM;
+        hipLaunchKernelGGL(fn, dim3(n_qt, d->B * d->H), dim3(kAttnThreads), lds, (hipStream_t)stream, ap);
+        return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
+    }
+    SplitPlan sp = plan_split(d);
+    if (!scratch) { sp.n_full = sp.n_pairs; sp.n_rem = 0; sp.splits = 1; }
+    ap.n_qt = sp.n_qt; ap.n_full = sp.n_full; ap.n_rem = sp.n_rem; ap.splits = sp.splits;
+    if (sp.splits > 1) {
+        const size_t slots = (size_t)sp.n_rem * sp.splits;
+        ap.part_acc = (float*)scratch;
+        ap.part_ml = (float2*)((char*)scratch + align256(slots * kSymBlockM * d->d_v * sizeof(float)));
+    }
+    const int64_t blocks = (int64_t)sp.n_full + (int64_t)sp.n_rem * sp.splits;
+    hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3(64 * kSymWaves), lds, (hipStream_t)stream, ap);
+    if (hipGetLastError() != hipSuccess) return COSMOS_ATTN_LAUNCH_FAILED;
+    if (sp.splits > 1) {
+        const int rows_per_block = 256 / (d->d_v / 4);
+        const int64_t rows = (int64_t)sp.n_rem * kSymBlockM;
+        const unsigned cblocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
+        if (d->dtype == COSMOS_ATTN_BF16)
+            hipLaunchKernelGGL(attn_combine_kernel<__bf16>, dim3(cblocks), dim3(256), 0, (hipStream_t)stream, ap, d->d_v);
+        else
+            hipLaunchKernelGGL(attn_combine_kernel<_Float16>, dim3(cblocks), dim3(256), 0, (hipStream_t)stream, ap, d->d_v);
+        if (hipGetLastError() != hipSuccess) return COSMOS_ATTN_LAUNCH_FAILED;
+    }
+    return COSMOS_ATTN_OK;
+}
+}  // namespace
+
+extern "C" {
+
+COSMOS_ATTN_API int cosmos_attn_run(const cosmos_attn_desc* d, const void* workspace, size_t workspace_bytes, void* stream) {
+    return run_impl(d, workspace, workspace_bytes, nullptr, stream);
 }
 
 COSMOS_ATTN_API int cosmos_attn_fwd_jvp(const cosmos_attn_desc* d, void* workspace, size_t workspace_bytes, void* stream) {
     const int st = cosmos_attn_pack_kv(d, workspace, workspace_bytes, stream);
     if (st != COSMOS_ATTN_OK) return st;
-    return cosmos_attn_run(d, workspace, workspace_bytes, stream);
+    void* scratch = partial_bytes_of(d) ? (char*)workspace + align256(tiles_bytes_of(d)) : nullptr;
+    return run_impl(d, workspace, workspace_bytes, scratch, stream);
 }
 
 }  // extern "C"

@@ -106,6 +106,44 @@ def test_forward_only_key_padding(pkg, oracle, gpu, lens):
     run_case(pkg, oracle, gpu, (2, 2, 450, 128), (2, 2, 512, 128), key_lens=lens, seed=sum(lens), tangents="none")
 
 
+@pytest.mark.parametrize("shape_q,Lkv,ranges", [
+    ((1, 2, 1000, 128), 1000, 4),      # 6 workgroup pairs, 16 steps of 64 keys: 4 key ranges each
+    ((1, 1, 1157, 32), 4000, 15),      # 4 pairs, 63 steps: 15 ranges of 4 or 5 steps
+    ((1, 3, 300, 128), 520, 2),        # 3 pairs, 9 steps: 2 ranges (4 + 5 steps); ragged last tile in the second
+    ((2, 8, 6500, 64), 700, 2),        # 272 pairs: 256 whole + 16 cut into ... 11 steps allow 2 ranges
+    ((1, 2, 400, 64), 250, 1),         # 4 steps only: too short to cut
+])
+def test_forward_only_key_range_split(pkg, oracle, gpu, shape_q, Lkv, ranges):
+    """When the last round of forward-only workgroups (one per compute unit) is less than half full, its (query block,
+    head) pairs are cut along the keys and merged by a second kernel.  The one-call entry point (which may cut) and
+    pack + run (which never does) must agree to rounding, and both with the oracle."""
+    del ranges   # documented above; the plan itself is internal
+    B, H, Lq, d = shape_q
+    run_case(pkg, oracle, gpu, shape_q, (B, H, Lkv, d), seed=Lq + Lkv, tangents="none")
+    L, lib = pkg._lib, pkg._lib.load_library()
+    q, k, v, _, _, _ = (x.to(gpu) for x in oracle.make_inputs(shape_q, (B, H, Lkv, d), seed=Lq + Lkv))
+    o_ref, _, lse_ref = pkg.fwd_jvp(q, k, v)
+    o, lse = torch.empty_like(q), torch.empty(B, H, Lq, device=gpu)
+    D = L.AttnDesc()
+    D.abi_version, D.dtype = L.ABI_VERSION, L.DTYPE_BF16
+    D.B, D.H, D.Lq, D.Lkv, D.d_qk, D.d_v, D.causal, D.sm_scale = B, H, Lq, Lkv, d, d, 0, d ** -0.5
+    D.q, D.k, D.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    s3 = lambda x: (ctypes.c_int64 * 3)(x.stride(0), x.stride(1), x.stride(2))
+    D.q_stride, D.k_stride, D.v_stride, D.o_stride = s3(q), s3(k), s3(v), s3(o)
+    D.o, D.lse = o.data_ptr(), lse.data_ptr()
+    n = lib.cosmos_attn_workspace_bytes(ctypes.byref(D))
+    ws = torch.empty(n, device=gpu, dtype=torch.uint8)
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.cosmos_attn_pack_kv(ctypes.byref(D), ws.data_ptr(), n, st) == 0
+    assert lib.cosmos_attn_run(ctypes.byref(D), ws.data_ptr(), n, st) == 0
+    torch.cuda.synchronize()
+    assert float((o.float() - o_ref.float()).abs().max()) <= 2.0 ** -7 * max(1.0, float(o_ref.float().abs().max()))
+    assert float((lse - lse_ref).abs().max()) <= 1e-4
+    # same inputs, same plan: bitwise repeatable
+    o_again, _, lse_again = pkg.fwd_jvp(q, k, v)
+    assert torch.equal(o_again, o_ref) and torch.equal(lse_again, lse_ref)
+
+
 def test_against_torch_sdpa_jvp(pkg, oracle, gpu):
     """The quoted oracle itself (torch math SDPA under torch.func.jvp, fp32) on a mid-size case."""
     q, k, v, tq, tk, tv = oracle.make_inputs((2, 3, 300, 128), seed=5)
@@ -327,7 +365,7 @@ def test_golden_fixtures(pkg, oracle, gpu):
         assert oracle.error_metrics(lse.cpu(), gold[name + "/lse"])[0] <= LSE_ABS
 
 
-# ------------------------------------------------------------------ BASELINE shapes: sampled row blocks + size-independent properties
+# ------------------------------------------------------------------ the benchmark shapes: sampled row blocks + size-independent properties
 def sampled_rows_check(pkg, oracle, gpu, H, Lq, Lkv, tangents, rms, key_lens=None, B=1, seed=0, n_blocks=8):
     """Full-length sequences: the fp32 score matrix cannot exist, so 128-row blocks (first, last / ragged, random) of a
     couple of heads are checked against the row-block oracle -- exact, because query rows are independent."""
@@ -357,7 +395,7 @@ def sampled_rows_check(pkg, oracle, gpu, H, Lq, Lkv, tangents, rms, key_lens=Non
 
 
 def test_config3_shape_2b_720p_fwd_jvp(pkg, oracle, gpu):
-    """BASELINE config 3 at its real sequence length (L=84480, d=128, bf16, primals N(0,1), tangents N(0,1)*0.1) on 2 of
+    """The 2B 720p forward + JVP configuration at its real sequence length (L=84480, d=128, bf16, primals N(0,1), tangents N(0,1)*0.1) on 2 of
     the 16 heads (heads are independent; the full-H run is bench.py's), plus properties that need no oracle."""
     (q, k, v, tq, tk, tv), (o, to, lse) = sampled_rows_check(pkg, oracle, gpu, H=2, Lq=84480, Lkv=84480, tangents="full", rms=False)
     dq, dk, dv, dtq, dtk, dtv = (x.to(gpu) for x in (q, k, v, tq, tk, tv))
@@ -387,17 +425,17 @@ def test_config3_shape_2b_720p_fwd_jvp(pkg, oracle, gpu):
 
 
 def test_config2_shape_480p_forward_ragged(pkg, oracle, gpu):
-    """BASELINE config 2: L=37440 (not a multiple of 128 or 64), forward only, RMS-normed q/k, LSE returned."""
+    """The 2B 480p forward-only configuration: L=37440 (not a multiple of 128 or 64), forward only, RMS-normed q/k, LSE returned."""
     sampled_rows_check(pkg, oracle, gpu, H=2, Lq=37440, Lkv=37440, tangents="none", rms=True, seed=1)
 
 
 def test_config4_shape_14b_rms_normed(pkg, oracle, gpu):
-    """BASELINE config 4 differs from config 3 in H=40 and RMS-normed q/k: 3 heads at L=84480."""
+    """The 14B configuration differs from the 2B 720p one in H=40 and RMS-normed q/k: 3 heads at L=84480."""
     sampled_rows_check(pkg, oracle, gpu, H=3, Lq=84480, Lkv=84480, tangents="full", rms=True, seed=2, n_blocks=4)
 
 
 def test_config5_shape_cross_attention_key_padding(pkg, oracle, gpu):
-    """BASELINE config 5: B=2, Lq=37440, Lkv=512, per-row key lengths in 64..512, tangent on q only."""
+    """The text cross-attention configuration: B=2, Lq=37440, Lkv=512, per-row key lengths in 64..512, tangent on q only."""
     g = torch.Generator().manual_seed(0)
     lens = [int(x) for x in torch.randint(64, 513, (2,), generator=g)]
     (q, k, v, tq, _, _), (o, to, lse) = sampled_rows_check(pkg, oracle, gpu, H=4, Lq=37440, Lkv=512, tangents="q", rms=False, key_lens=lens, B=2, seed=3)

@@ -57,7 +57,7 @@ def test_sdpa_jvp_wrapper_matches_closed_form_fp32(oracle):
 
 
 def test_config1_fp32_plumbing_within_1e5(oracle):
-    """BASELINE config 1: B1 H16 L2048 d128 fp32, N(0,1)*0.5, scale 1/sqrt(128): torch math SDPA + jvp (fp32) against
+    """The CPU plumbing configuration: B1 H16 L2048 d128 fp32, N(0,1)*0.5, scale 1/sqrt(128): torch math SDPA + jvp (fp32) against
     the fp64 closed form, tolerance 1e-5 (4 heads are checked in fp64 to keep the CPU suite short)."""
     q, k, v, tq, tk, tv = oracle.make_inputs((1, 16, 2048, 128), seed=0, primal_std=0.5, tangent_std=0.5, dtype=torch.float32)
     o, to = oracle.sdpa_jvp_torch(q, k, v, tq, tk, tv)
