@@ -135,11 +135,12 @@ struct AttnParams {
     const int32_t* key_lens;   // nullable
     int H, Lq, Lkv, n_tiles, causal;
     float sm_scale, scale_log2;
-    // forward-only kernel: workgroups [0, n_full) each own a (query block, head) pair; the remaining pairs are cut into
-    // `splits` key ranges, one workgroup each, which leave unnormalised partial results for attn_combine_kernel
+    // 1-D grid: workgroups [0, n_full) each own a (query block, head) pair; the remaining n_rem pairs are cut into
+    // `splits` key ranges, one workgroup each, which leave unnormalised partial results for attn_combine_kernel.
+    // slot = (pair - n_full) * splits + split; block_m = query rows per workgroup (128, or 384 forward only)
     int n_qt, n_full, n_rem, splits;
-    float* part_acc;           // [(pair - n_full) * splits + split][kSymBlockM][d_v]
-    float2* part_ml;           // same leading index, [kSymBlockM]: (running max in log2 units, row sum)
+    float* part_acc;           // [slot][block_m][d_v] accumulators; with tangents [slot][block_m][2][d_v] (O, T)
+    float4* part_stat;         // [slot][block_m]: (running max in log2 units, row sum of P, row sum of H, 0)
 };
 
 extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -389,7 +390,12 @@ attn_fwd_jvp_kernel(const AttnParams p) {
     constexpr int IN_FLIGHT = 2 * C::KP_LOADS + C::VP_LOADS;
     constexpr int WAIT_FILLS = (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14) | 0x0F70;
 
-    const int qt = blockIdx.x, bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
+    // 1-D grid: block id -> (pair, key range); pair = query block + n_qt * (batch * H + head)
+    const int bid = blockIdx.x;
+    const bool partial = bid >= p.n_full && p.splits > 1;
+    const int pair = partial ? p.n_full + (bid - p.n_full) / p.splits : bid;
+    const int split = partial ? (bid - p.n_full) % p.splits : 0;
+    const int qt = pair % p.n_qt, bh = pair / p.n_qt, b = bh / p.H, h = bh % p.H;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const bool score_role = wave < 4;            // wavefronts w and w + 4 (same SIMD) serve query rows 32 w .. 32 w + 31
@@ -400,8 +406,11 @@ attn_fwd_jvp_kernel(const AttnParams p) {
 
     int kv_len = p.Lkv;
     if (p.key_lens) { const int kl = p.key_lens[b]; kv_len = kl < kv_len ? (kl < 0 ? 0 : kl) : kv_len; }
-    int n_tiles = (kv_len + kBlockN - 1) / kBlockN;
-    if (p.causal) { const int lim = (qt * kBlockM + kBlockM + kBlockN - 1) / kBlockN; n_tiles = n_tiles < lim ? n_tiles : lim; }
+    int n_tiles_all = (kv_len + kBlockN - 1) / kBlockN;
+    if (p.causal) { const int lim = (qt * kBlockM + kBlockM + kBlockN - 1) / kBlockN; n_tiles_all = n_tiles_all < lim ? n_tiles_all : lim; }
+    // this workgroup's share of the sweep: positions [u_lo, u_lo + n_tiles)  (the whole sweep unless the pair is cut)
+    const int u_lo = partial ? (int)((int64_t)split * n_tiles_all / p.splits) : 0;
+    const int n_tiles = partial ? (int)((int64_t)(split + 1) * n_tiles_all / p.splits) - u_lo : n_tiles_all;
 
     char* const kring = smem + C::KRING_OFF;
     char* const vring = smem + C::VRING_OFF;
@@ -413,12 +422,11 @@ attn_fwd_jvp_kernel(const AttnParams p) {
     // that share one XCD's L2 (workgroup ids congruent mod 8) start a few tiles apart, so that the first one to
     // reach a tile takes the L2 miss and the ones behind it hit.  The shift is a fixed function of the workgroup id:
     // results are bitwise reproducible from run to run.
-    const int n_sweep = n_tiles > 0 ? n_tiles : 1;
-    const int wg_linear = blockIdx.x + gridDim.x * blockIdx.y;
+    const int n_sweep = n_tiles_all > 0 ? n_tiles_all : 1;
     // (not with causal masking: there the first tile of the sweep must be tile 0, the one tile in which every query row
     // sees a key, so that the running max is finite from the first step on)
-    const int shift = p.causal ? 0 : (((wg_linear >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
-    auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane((u + shift) % n_sweep); };
+    const int shift = p.causal ? 0 : (((pair >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
+    auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane((u_lo + u + shift) % n_sweep); };
     auto wrap_inc = [&](int t) { ++t; return t >= n_sweep ? t - n_sweep : t; };
     const int k_run = ((qw * C::KP_LOADS) % C::KP_FR) * kFragBytes, v_run = ((qw * C::VP_LOADS) % C::VP_FR) * kFragBytes;
     // tk / tv: tiles whose K part / V part the group copies; ku / vu: sweep positions that pick the ring slots
@@ -513,7 +521,14 @@ attn_fwd_jvp_kernel(const AttnParams p) {
         asm volatile("ds_write_b32 %0, %1" ::"v"(lds0 + alpha_base + 4 * 256 + 4 * lane), "v"(r_over_l) : "memory");
         __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
         __builtin_amdgcn_s_barrier();
-        if (row < p.Lq && p.lse && hh == 0) p.lse[(int64_t)bh * p.Lq + row] = (w.m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
+        if (partial) {   // a key range only: leave the statistics for attn_combine_kernel
+            if (hh == 0) {
+                const int64_t slot = (int64_t)(pair - p.n_full) * p.splits + split;
+                p.part_stat[slot * kBlockM + qw * 32 + j] = make_float4(w.m_run, l_tot, r_tot, 0.f);
+            }
+        } else if (row < p.Lq && p.lse && hh == 0) {
+            p.lse[(int64_t)bh * p.Lq + row] = (w.m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
+        }
     } else {
         OW w;
         w.lane = lane;
@@ -543,7 +558,21 @@ attn_fwd_jvp_kernel(const AttnParams p) {
         // ---- epilogue, outputs: O = acc / l ; dO = (T - (r / l) acc) / l ----
         const float inv_l = *reinterpret_cast<const float*>(smem + alpha_base + 4 * lane);
         const float r_over_l = *reinterpret_cast<const float*>(smem + alpha_base + 4 * 256 + 4 * lane);
-        if (row < p.Lq) {
+        if (partial) {   // a key range only: leave the unnormalised accumulators for attn_combine_kernel
+            const int64_t slot = (int64_t)(pair - p.n_full) * p.splits + split;
+            float* pa = p.part_acc + (slot * kBlockM + qw * 32 + j) * (JVP ? 2 * DV : DV);
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int d = 32 * db + 8 * g + 4 * hh;
+                    if (d < DV) {
+                        *reinterpret_cast<float4*>(pa + d) = make_float4(w.acc[db][4 * g], w.acc[db][4 * g + 1], w.acc[db][4 * g + 2], w.acc[db][4 * g + 3]);
+                        if (JVP) *reinterpret_cast<float4*>(pa + DV + d) = make_float4(w.acct[db][4 * g], w.acct[db][4 * g + 1], w.acct[db][4 * g + 2], w.acct[db][4 * g + 3]);
+                    }
+                }
+            }
+        } else if (row < p.Lq) {
             const int64_t off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)row * p.o_sl;
             T* op = reinterpret_cast<T*>(p.o) + off;
             T* top = reinterpret_cast<T*>(p.to) + off;
@@ -829,7 +858,7 @@ attn_fwd_sym_kernel(const AttnParams p) {
                     *reinterpret_cast<float4*>(pa + d) = make_float4(w.acc[db][4 * g], w.acc[db][4 * g + 1], w.acc[db][4 * g + 2], w.acc[db][4 * g + 3]);
             }
         }
-        if (hh == 0) p.part_ml[slot * kSymBlockM + wrow] = make_float2(w.m_run, l_tot);
+        if (hh == 0) p.part_stat[slot * kSymBlockM + wrow] = make_float4(w.m_run, l_tot, 0.f, 0.f);
         return;
     }
     const float inv_l = 1.0f / l_tot;
@@ -853,34 +882,50 @@ attn_fwd_sym_kernel(const AttnParams p) {
 }
 
 // Merge the key-range partial results of one query row:  M = max m_i,  w_i = 2^(m_i - M),  L = sum l_i w_i,
-// O = sum acc_i w_i / L,  LSE = (M + log2 L) ln 2.  One thread per (row, 4 output channels); fixed order over the ranges.
-template <typename T>
-__global__ void __launch_bounds__(256) attn_combine_kernel(const AttnParams p, int dv) {
+// O = sum acc_i w_i / L,  LSE = (M + log2 L) ln 2; with tangents also T = sum accT_i w_i, R = sum r_i w_i and
+// dO = (T - (R / L) sum acc_i w_i) / L.  One thread per (row, 4 output channels); fixed order over the ranges.
+template <typename T, bool JVP>
+__global__ void __launch_bounds__(256) attn_combine_kernel(const AttnParams p, int dv, int block_m) {
     typedef typename VecOf<T>::v4 V4;
     const int tpr = dv / 4;                                   // threads per row
     const int64_t r = (int64_t)blockIdx.x * (256 / tpr) + threadIdx.x / tpr;   // row among the split pairs' rows
     const int c = (threadIdx.x % tpr) * 4;
-    const int pair_i = (int)(r / kSymBlockM), wrow = (int)(r % kSymBlockM);
+    const int pair_i = (int)(r / block_m), wrow = (int)(r % block_m);
     const int pair = p.n_full + pair_i;
     const int qt = pair % p.n_qt, bh = pair / p.n_qt, b = bh / p.H, h = bh % p.H;
-    const int row = qt * kSymBlockM + wrow;
+    const int row = qt * block_m + wrow;
     if (pair_i >= p.n_rem || row >= p.Lq) return;
     const int64_t slot0 = (int64_t)pair_i * p.splits;
+    const int acc_w = JVP ? 2 * dv : dv;                      // floats per row in part_acc
     float M = -INFINITY;
-    for (int i = 0; i < p.splits; ++i) M = fmaxf(M, p.part_ml[(slot0 + i) * kSymBlockM + wrow].x);
-    float L = 0.f, o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+    for (int i = 0; i < p.splits; ++i) M = fmaxf(M, p.part_stat[(slot0 + i) * block_m + wrow].x);
+    float L = 0.f, R = 0.f;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f), t = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int i = 0; i < p.splits; ++i) {
-        const float2 ml = p.part_ml[(slot0 + i) * kSymBlockM + wrow];
-        const float wgt = __builtin_amdgcn_exp2f(ml.x - M);
-        const float4 a = *reinterpret_cast<const float4*>(p.part_acc + ((slot0 + i) * kSymBlockM + wrow) * dv + c);
-        L += ml.y * wgt;
-        o0 += a.x * wgt; o1 += a.y * wgt; o2 += a.z * wgt; o3 += a.w * wgt;
+        const float4 st = p.part_stat[(slot0 + i) * block_m + wrow];
+        const float wgt = __builtin_amdgcn_exp2f(st.x - M);
+        const float* pa = p.part_acc + ((slot0 + i) * block_m + wrow) * acc_w + c;
+        const float4 a = *reinterpret_cast<const float4*>(pa);
+        L += st.y * wgt;
+        o.x += a.x * wgt; o.y += a.y * wgt; o.z += a.z * wgt; o.w += a.w * wgt;
+        if (JVP) {
+            const float4 at = *reinterpret_cast<const float4*>(pa + dv);
+            R += st.z * wgt;
+            t.x += at.x * wgt; t.y += at.y * wgt; t.z += at.z * wgt; t.w += at.w * wgt;
+        }
     }
     const float inv_l = 1.0f / L;
-    T* op = reinterpret_cast<T*>(p.o) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)row * p.o_sl;
+    const int64_t off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)row * p.o_sl + c;
     V4 ov;
-    ov[0] = (T)(o0 * inv_l); ov[1] = (T)(o1 * inv_l); ov[2] = (T)(o2 * inv_l); ov[3] = (T)(o3 * inv_l);
-    *reinterpret_cast<V4*>(op + c) = ov;
+    ov[0] = (T)(o.x * inv_l); ov[1] = (T)(o.y * inv_l); ov[2] = (T)(o.z * inv_l); ov[3] = (T)(o.w * inv_l);
+    *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.o) + off) = ov;
+    if (JVP) {
+        const float r_over_l = R * inv_l;
+        V4 tv;
+        tv[0] = (T)((t.x - r_over_l * o.x) * inv_l); tv[1] = (T)((t.y - r_over_l * o.y) * inv_l);
+        tv[2] = (T)((t.z - r_over_l * o.z) * inv_l); tv[3] = (T)((t.w - r_over_l * o.w) * inv_l);
+        *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.to) + off) = tv;
+    }
     if (p.lse && c == 0) p.lse[(int64_t)bh * p.Lq + row] = (M + __builtin_log2f(L)) * 0.6931471805599453f;
 }
 
@@ -944,21 +989,23 @@ int n_tiles_of(const cosmos_attn_desc* d) { return (d->Lkv + kBlockN - 1) / kBlo
 // workspace = packed tiles [B*H][n_tiles][tile bytes]
 size_t tiles_bytes_of(const cosmos_attn_desc* d) { return (size_t)d->B * d->H * n_tiles_of(d) * tile_bytes_of(d); }
 
-// Forward only: how the (query block, head) pairs are dealt out.  One workgroup fits on a compute unit, so a launch
-// runs in rounds of kNumCUs workgroups; when the last round is less than half full its pairs are cut along the keys
-// into as many ranges as fill it, and a small second kernel merges the ranges.
+// How the (query block, head) pairs are dealt out.  One workgroup fits on a compute unit, so a launch runs in rounds of
+// kNumCUs workgroups; when the last round is less than half full its pairs are cut along the keys into as many ranges
+// as fill it, and a small second kernel merges the ranges.
 constexpr int kNumCUs = 256;
 constexpr int kMaxSplits = 16;
-constexpr int kMinStepsPerSplit = 4;
-struct SplitPlan { int n_qt, n_pairs, n_full, n_rem, splits; };
+constexpr int kMinStepsPerSplit = 4;      // in barrier steps: 64 keys forward only, 32 keys with tangents
+struct SplitPlan { int block_m, n_qt, n_pairs, n_full, n_rem, splits; };
 SplitPlan plan_split(const cosmos_attn_desc* d) {
     SplitPlan s;
-    s.n_qt = (d->Lq + kSymBlockM - 1) / kSymBlockM;
+    const bool fwd = mode_of(d) == MODE_FWD;
+    s.block_m = fwd ? kSymBlockM : kBlockM;
+    s.n_qt = (d->Lq + s.block_m - 1) / s.block_m;
     s.n_pairs = s.n_qt * d->B * d->H;
     s.n_rem = 0; s.splits = 1; s.n_full = s.n_pairs;
     if (d->causal || d->key_lens) return s;          // key ranges of equal work only
     const int rem = s.n_pairs % kNumCUs;
-    const int n_steps = (n_tiles_of(d) + 1) / 2;
+    const int n_steps = fwd ? (n_tiles_of(d) + 1) / 2 : n_tiles_of(d);
     if (rem == 0 || rem > kNumCUs / 2) return s;
     int splits = kNumCUs / rem;
     if (splits > kMaxSplits) splits = kMaxSplits;
@@ -968,13 +1015,15 @@ SplitPlan plan_split(const cosmos_attn_desc* d) {
     return s;
 }
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
-// partial results of the split pairs: fp32 accumulators [slots][kSymBlockM][d_v], then (max, sum) [slots][kSymBlockM]
+// partial results of the split pairs: fp32 accumulators (O, and T with tangents), then the row statistics
+size_t partial_acc_bytes(const cosmos_attn_desc* d, const SplitPlan& s) {
+    const size_t per_row = (size_t)d->d_v * (mode_of(d) == MODE_FWD ? 1 : 2) * sizeof(float);
+    return align256((size_t)s.n_rem * s.splits * s.block_m * per_row);
+}
 size_t partial_bytes_of(const cosmos_attn_desc* d) {
-    if (mode_of(d) != MODE_FWD) return 0;
     const SplitPlan s = plan_split(d);
     if (s.splits < 2) return 0;
-    const size_t slots = (size_t)s.n_rem * s.splits;
-    return align256(slots * kSymBlockM * d->d_v * sizeof(float)) + align256(slots * kSymBlockM * sizeof(float2));
+    return partial_acc_bytes(d, s) + align256((size_t)s.n_rem * s.splits * s.block_m * sizeof(float4));
 }
 
 int validate(const cosmos_attn_desc* d) {
@@ -996,7 +1045,7 @@ int validate(const cosmos_attn_desc* d) {
         return COSMOS_ATTN_BAD_STRIDE;
     if (!strides_ok(d->q_stride) || !strides_ok(d->k_stride) || !strides_ok(d->v_stride) || !strides_ok(d->o_stride))
         return COSMOS_ATTN_BAD_STRIDE;
-    if ((int64_t)d->B * d->H > 65535) return COSMOS_ATTN_BAD_SHAPE;   // grid.y limit
+    if ((int64_t)d->B * d->H * ((d->Lq + kBlockM - 1) / kBlockM) > ((int64_t)1 << 30)) return COSMOS_ATTN_BAD_SHAPE;   // 1-D grid, 32-bit pair index
     if ((int64_t)n_tiles_of(d) * (int64_t)tile_bytes_of(d) >= (int64_t)1 << 31) return COSMOS_ATTN_BAD_SHAPE;   // 32-bit buffer offsets per head
     return COSMOS_ATTN_OK;
 }
@@ -1012,7 +1061,7 @@ COSMOS_ATTN_API const char* cosmos_attn_status_string(int status) {
     switch (status) {
         case COSMOS_ATTN_OK: return "ok";
         case COSMOS_ATTN_BAD_ARG: return "bad argument (null pointer, non-positive size, ABI version, or tangent set other than none / q only / q,k,v)";
-        case COSMOS_ATTN_BAD_SHAPE: return "bad shape (head dims must be in {16,32,64,128}; causal needs Lq == Lkv; B*H <= 65535)";
+        case COSMOS_ATTN_BAD_SHAPE: return "bad shape (head dims must be in {16,32,64,128}; causal needs Lq == Lkv)";
         case COSMOS_ATTN_BAD_STRIDE: return "bad stride or alignment (16-byte aligned bases, strides multiple of 8 elements, innermost stride 1)";
         case COSMOS_ATTN_UNSUPPORTED: return "unsupported dtype or head dim (bf16/fp16, head dim <= 128)";
         case COSMOS_ATTN_WORKSPACE_TOO_SMALL: return "workspace too small or null";
@@ -1067,31 +1116,25 @@ int run_impl(const cosmos_attn_desc* d, const void* workspace, size_t workspace_
     ap.sm_scale = d->sm_scale; ap.scale_log2 = d->sm_scale * 1.4426950408889634f;
     const size_t lds = lds_bytes_of(d);
     if (!allow_lds((const void*)fn, lds)) return COSMOS_ATTN_LAUNCH_FAILED;
-    ap.n_qt = 0; ap.n_full = 0; ap.n_rem = 0; ap.splits = 1; ap.part_acc = nullptr; ap.part_ml = nullptr;
-    if (mode != MODE_FWD) {
-        const int n_qt = (d->Lq + kBlockM - 1) / kBlockM;
-        hipLaunchKernelGGL(fn, dim3(n_qt, d->B * d->H), dim3(kAttnThreads), lds, (hipStream_t)stream, ap);
-        return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
-    }
     SplitPlan sp = plan_split(d);
     if (!scratch) { sp.n_full = sp.n_pairs; sp.n_rem = 0; sp.splits = 1; }
     ap.n_qt = sp.n_qt; ap.n_full = sp.n_full; ap.n_rem = sp.n_rem; ap.splits = sp.splits;
+    ap.part_acc = nullptr; ap.part_stat = nullptr;
     if (sp.splits > 1) {
-        const size_t slots = (size_t)sp.n_rem * sp.splits;
         ap.part_acc = (float*)scratch;
-        ap.part_ml = (float2*)((char*)scratch + align256(slots * kSymBlockM * d->d_v * sizeof(float)));
+        ap.part_stat = (float4*)((char*)scratch + partial_acc_bytes(d, sp));
     }
     const int64_t blocks = (int64_t)sp.n_full + (int64_t)sp.n_rem * sp.splits;
-    hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3(64 * kSymWaves), lds, (hipStream_t)stream, ap);
+    hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3(mode == MODE_FWD ? 64 * kSymWaves : kAttnThreads), lds, (hipStream_t)stream, ap);
     if (hipGetLastError() != hipSuccess) return COSMOS_ATTN_LAUNCH_FAILED;
     if (sp.splits > 1) {
         const int rows_per_block = 256 / (d->d_v / 4);
-        const int64_t rows = (int64_t)sp.n_rem * kSymBlockM;
-        const unsigned cblocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
-        if (d->dtype == COSMOS_ATTN_BF16)
-            hipLaunchKernelGGL(attn_combine_kernel<__bf16>, dim3(cblocks), dim3(256), 0, (hipStream_t)stream, ap, d->d_v);
-        else
-            hipLaunchKernelGGL(attn_combine_kernel<_Float16>, dim3(cblocks), dim3(256), 0, (hipStream_t)stream, ap, d->d_v);
+        const int64_t rows = (int64_t)sp.n_rem * sp.block_m;
+        const dim3 cgrid((unsigned)((rows + rows_per_block - 1) / rows_per_block));
+        const bool bf16 = d->dtype == COSMOS_ATTN_BF16, jvp = mode != MODE_FWD;
+        auto cfn = jvp ? (bf16 ? attn_combine_kernel<__bf16, true> : attn_combine_kernel<_Float16, true>)
+                       : (bf16 ? attn_combine_kernel<__bf16, false> : attn_combine_kernel<_Float16, false>);
+        hipLaunchKernelGGL(cfn, cgrid, dim3(256), 0, (hipStream_t)stream, ap, d->d_v, sp.block_m);
         if (hipGetLastError() != hipSuccess) return COSMOS_ATTN_LAUNCH_FAILED;
     }
     return COSMOS_ATTN_OK;
