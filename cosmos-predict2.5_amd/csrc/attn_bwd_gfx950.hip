@@ -180,6 +180,10 @@ struct BwdParams {
     const char* stream;                // packed stream tiles [B*H][n_tiles][tile bytes]
     int H, L_stat, L_stream, n_tiles, causal;
     float sm_scale, scale_log2;
+    // 1-D grid: workgroups [0, n_full) each own a (block of 128 stationary rows, head) pair; the remaining n_rem pairs
+    // are cut into `splits` ranges of the stream, one workgroup each, which leave fp32 partial sums for bwd_combine_kernel
+    int n_blk, n_full, n_rem, splits;
+    float* part;                       // [(pair - n_full) * splits + split][kBlock][D] (dQ) or [..][kBlock][2][D] (dV, dK)
 };
 
 extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -343,7 +347,11 @@ attn_bwd_kernel(const BwdParams p) {
     constexpr int IN_FLIGHT = 2 * (C::SP_LOADS + C::ST_FR) + C::OP_LOADS;
     constexpr int WAIT_FILLS = (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14) | 0x0F70;
 
-    const int blk = blockIdx.x, bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
+    const int bid = blockIdx.x;
+    const bool partial = bid >= p.n_full && p.splits > 1;
+    const int pair = partial ? p.n_full + (bid - p.n_full) / p.splits : bid;
+    const int split = partial ? (bid - p.n_full) % p.splits : 0;
+    const int blk = pair % p.n_blk, bh = pair / p.n_blk, b = bh / p.H, h = bh % p.H;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const bool score_role = wave < 4;            // wavefronts w and w + 4 (same SIMD) serve stationary rows 32 w .. 32 w + 31
@@ -360,6 +368,11 @@ attn_bwd_kernel(const BwdParams p) {
         if (DKDV) t_lo = (blk * kBlock) / kRows;
         else { const int lim = (blk * kBlock + kBlock + kRows - 1) / kRows; t_hi = t_hi < lim ? t_hi : lim; }
     }
+    if (partial) {   // this workgroup's range of the stream (never with causal masking)
+        const int n = p.n_tiles;
+        t_lo = (int)((int64_t)split * n / p.splits);
+        t_hi = (int)((int64_t)(split + 1) * n / p.splits);
+    }
     const int n_steps = t_hi > t_lo ? t_hi - t_lo : 0;
 
     char* const sring = smem + C::SRING_OFF;
@@ -370,8 +383,7 @@ attn_bwd_kernel(const BwdParams p) {
     // Sweep order: accumulation is order-free, so workgroups that share an XCD's L2 start a few tiles apart and wrap
     // around (a fixed function of the workgroup id: results stay bitwise reproducible).
     const int n_sweep = n_steps > 0 ? n_steps : 1;
-    const int wg_linear = blockIdx.x + gridDim.x * blockIdx.y;
-    const int shift = (((wg_linear >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
+    const int shift = (((pair >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
     auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane(t_lo + (u + shift) % n_sweep); };
     auto wrap_inc = [&](int t) { ++t; return t >= t_lo + n_sweep ? t - n_sweep : t; };
     const int s_run = ((qw * C::SP_LOADS) % C::SP_FR) * kFragBytes, o_run = ((qw * C::OP_LOADS) % C::OP_FR) * kFragBytes;
@@ -480,7 +492,21 @@ attn_bwd_kernel(const BwdParams p) {
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);   // drain the (unused) trailing fills before the LDS is released
         // ---- epilogue: dQ = s dQ^T   |   dV = dV^T, dK = s dK^T ----
-        if (row < p.L_stat) {
+        if (partial) {   // a range of the stream only: leave the sums for bwd_combine_kernel
+            const int64_t slot = (int64_t)(pair - p.n_full) * p.splits + split;
+            float* pa = p.part + (slot * kBlock + qw * kRows + j) * (DKDV ? 2 * D : D);
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int d = 32 * db + 8 * g + 4 * hh;
+                    if (d < D) {
+                        *reinterpret_cast<float4*>(pa + d) = make_float4(w.acc1[db][4 * g], w.acc1[db][4 * g + 1], w.acc1[db][4 * g + 2], w.acc1[db][4 * g + 3]);
+                        if (DKDV) *reinterpret_cast<float4*>(pa + D + d) = make_float4(w.acc2[db][4 * g], w.acc2[db][4 * g + 1], w.acc2[db][4 * g + 2], w.acc2[db][4 * g + 3]);
+                    }
+                }
+            }
+        } else if (row < p.L_stat) {
             T* o1 = reinterpret_cast<T*>(p.out1) + (int64_t)b * p.o1_sb + (int64_t)h * p.o1_sh + (int64_t)row * p.o1_sl;
             T* o2 = DKDV ? reinterpret_cast<T*>(p.out2) + (int64_t)b * p.o2_sb + (int64_t)h * p.o2_sh + (int64_t)row * p.o2_sl : nullptr;
             const float s1 = DKDV ? 1.0f : p.sm_scale;
@@ -502,6 +528,41 @@ attn_bwd_kernel(const BwdParams p) {
                 }
             }
         }
+    }
+}
+
+// Add the partial sums of the ranges of one stationary row (fixed order), scale, round, store.
+// One thread per (row, 4 channels).
+template <typename T, bool DKDV>
+__global__ void __launch_bounds__(256) bwd_combine_kernel(const BwdParams p, int D) {
+    typedef typename VecOf<T>::v4 V4;
+    const int tpr = D / 4;
+    const int64_t r = (int64_t)blockIdx.x * (256 / tpr) + threadIdx.x / tpr;
+    const int c = (threadIdx.x % tpr) * 4;
+    const int pair_i = (int)(r / kBlock), wrow = (int)(r % kBlock);
+    const int pair = p.n_full + pair_i;
+    const int blk = pair % p.n_blk, bh = pair / p.n_blk, b = bh / p.H, h = bh % p.H;
+    const int row = blk * kBlock + wrow;
+    if (pair_i >= p.n_rem || row >= p.L_stat) return;
+    const int W = DKDV ? 2 * D : D;
+    float4 a1 = make_float4(0.f, 0.f, 0.f, 0.f), a2 = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = 0; i < p.splits; ++i) {
+        const float* pa = p.part + (((int64_t)pair_i * p.splits + i) * kBlock + wrow) * W + c;
+        const float4 x = *reinterpret_cast<const float4*>(pa);
+        a1.x += x.x; a1.y += x.y; a1.z += x.z; a1.w += x.w;
+        if (DKDV) {
+            const float4 y = *reinterpret_cast<const float4*>(pa + D);
+            a2.x += y.x; a2.y += y.y; a2.z += y.z; a2.w += y.w;
+        }
+    }
+    const float s1 = DKDV ? 1.0f : p.sm_scale;
+    V4 v1;
+    v1[0] = (T)(a1.x * s1); v1[1] = (T)(a1.y * s1); v1[2] = (T)(a1.z * s1); v1[3] = (T)(a1.w * s1);
+    *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.out1) + (int64_t)b * p.o1_sb + (int64_t)h * p.o1_sh + (int64_t)row * p.o1_sl + c) = v1;
+    if (DKDV) {
+        V4 v2;
+        v2[0] = (T)(a2.x * p.sm_scale); v2[1] = (T)(a2.y * p.sm_scale); v2[2] = (T)(a2.z * p.sm_scale); v2[3] = (T)(a2.w * p.sm_scale);
+        *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.out2) + (int64_t)b * p.o2_sb + (int64_t)h * p.o2_sh + (int64_t)row * p.o2_sl + c) = v2;
     }
 }
 
@@ -538,7 +599,31 @@ struct BwdGeom {
         stats_bytes = ((bh * d->Lq * sizeof(float2)) + 1023) / 1024 * 1024;
         q_img_bytes = bh * n_q_tiles * q_tile_bytes;
         k_img_bytes = bh * n_k_tiles * k_tile_bytes;
+        dkdv = plan((d->Lkv + kBlock - 1) / kBlock, (int)bh, n_q_tiles, d->causal != 0);
+        dq = plan((d->Lq + kBlock - 1) / kBlock, (int)bh, n_k_tiles, d->causal != 0);
+        const size_t p1 = (size_t)dkdv.n_rem * dkdv.splits * kBlock * 2 * d->d * sizeof(float);
+        const size_t p2 = (size_t)dq.n_rem * dq.splits * kBlock * d->d * sizeof(float);
+        part_bytes = ((p1 > p2 ? p1 : p2) + 1023) / 1024 * 1024;     // the two kernels run one after the other
     }
+    // How the (block of stationary rows, head) pairs of a kernel are dealt out.  One workgroup fits on a compute unit, so
+    // a launch runs in rounds of kNumCUs; when the last round is less than half full its pairs are cut along the stream
+    // into as many ranges as fill it, and bwd_combine_kernel adds the ranges up.
+    struct Plan { int n_blk, n_pairs, n_full, n_rem, splits; };
+    static Plan plan(int n_blk, int bh, int n_stream_tiles, bool causal) {
+        constexpr int kNumCUs = 256, kMaxSplits = 16, kMinStepsPerSplit = 4;
+        Plan s;
+        s.n_blk = n_blk; s.n_pairs = n_blk * bh; s.n_full = s.n_pairs; s.n_rem = 0; s.splits = 1;
+        const int rem = s.n_pairs % kNumCUs;
+        if (causal || rem == 0 || rem > kNumCUs / 2) return s;
+        int splits = kNumCUs / rem;
+        if (splits > kMaxSplits) splits = kMaxSplits;
+        if (splits > n_stream_tiles / kMinStepsPerSplit) splits = n_stream_tiles / kMinStepsPerSplit;
+        if (splits < 2) return s;
+        s.n_rem = rem; s.n_full = s.n_pairs - rem; s.splits = splits;
+        return s;
+    }
+    Plan dkdv, dq;
+    size_t part_bytes;
 };
 
 int validate_bwd(const cosmos_attn_bwd_desc* d) {
@@ -554,7 +639,7 @@ int validate_bwd(const cosmos_attn_bwd_desc* d) {
     for (const void* ptr : ptrs) if (!aligned16(ptr)) return COSMOS_ATTN_BAD_STRIDE;
     const int64_t* strides[] = {d->q_stride, d->k_stride, d->v_stride, d->o_stride, d->dout_stride, d->dq_stride, d->dk_stride, d->dv_stride};
     for (const int64_t* s : strides) if (!strides_ok(s)) return COSMOS_ATTN_BAD_STRIDE;
-    if ((int64_t)d->B * d->H > 65535) return COSMOS_ATTN_BAD_SHAPE;   // grid.y limit
+    if ((int64_t)d->B * d->H > 65535) return COSMOS_ATTN_BAD_SHAPE;   // grid.y limit of the re-tiling kernels
     const BwdGeom g(d);
     if ((int64_t)g.n_q_tiles * (int64_t)g.q_tile_bytes >= (int64_t)1 << 31) return COSMOS_ATTN_BAD_SHAPE;   // 32-bit buffer offsets per head
     if ((int64_t)g.n_k_tiles * (int64_t)g.k_tile_bytes >= (int64_t)1 << 31) return COSMOS_ATTN_BAD_SHAPE;
@@ -570,7 +655,7 @@ extern "C" {
 COSMOS_ATTN_API size_t cosmos_attn_bwd_workspace_bytes(const cosmos_attn_bwd_desc* d) {
     if (validate_bwd(d) != COSMOS_ATTN_OK) return 0;
     const BwdGeom g(d);
-    return g.stats_bytes + g.q_img_bytes + g.k_img_bytes;
+    return g.stats_bytes + g.q_img_bytes + g.k_img_bytes + g.part_bytes;
 }
 
 COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspace, size_t workspace_bytes, void* stream_) {
@@ -587,7 +672,21 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
     float2* stats = (float2*)ws;
     char* q_img = ws + g.stats_bytes;
     char* k_img = q_img + g.q_img_bytes;
+    float* part = (float*)(k_img + g.k_img_bytes);
     const int BH = d->B * d->H;
+    auto launch = [&](bwd_kernel_t fn, size_t lds, const BwdGeom::Plan& pl, BwdParams& bp, bool is_dkdv) {
+        bp.n_blk = pl.n_blk; bp.n_full = pl.n_full; bp.n_rem = pl.n_rem; bp.splits = pl.splits; bp.part = part;
+        if (!allow_lds((const void*)fn, lds)) return false;
+        hipLaunchKernelGGL(fn, dim3((unsigned)(pl.n_full + pl.n_rem * pl.splits)), dim3(kBwdThreads), lds, stream, bp);
+        if (pl.splits > 1) {
+            const int rows_per_block = 256 / (d->d / 4);
+            const dim3 cgrid((unsigned)(((int64_t)pl.n_rem * kBlock + rows_per_block - 1) / rows_per_block));
+            auto cfn = is_dkdv ? (bf16 ? bwd_combine_kernel<__bf16, true> : bwd_combine_kernel<_Float16, true>)
+                               : (bf16 ? bwd_combine_kernel<__bf16, false> : bwd_combine_kernel<_Float16, false>);
+            hipLaunchKernelGGL(cfn, cgrid, dim3(256), 0, stream, bp, d->d);
+        }
+        return true;
+    };
 
     {   // per-query statistics
         StatsParams sp;
@@ -626,8 +725,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
         bp.out1 = d->dv; bp.o1_sb = d->dv_stride[0]; bp.o1_sh = d->dv_stride[1]; bp.o1_sl = d->dv_stride[2];
         bp.out2 = d->dk; bp.o2_sb = d->dk_stride[0]; bp.o2_sh = d->dk_stride[1]; bp.o2_sl = d->dk_stride[2];
         bp.stream = q_img; bp.L_stat = d->Lkv; bp.L_stream = d->Lq; bp.n_tiles = g.n_q_tiles;
-        if (!allow_lds((const void*)k_dkdv, g.lds_dkdv)) return COSMOS_ATTN_LAUNCH_FAILED;
-        hipLaunchKernelGGL(k_dkdv, dim3((d->Lkv + kBlock - 1) / kBlock, BH), dim3(kBwdThreads), g.lds_dkdv, stream, bp);
+        if (!launch(k_dkdv, g.lds_dkdv, g.dkdv, bp, true)) return COSMOS_ATTN_LAUNCH_FAILED;
     }
     {   // dQ: stationary queries, streamed keys
         bp.st1 = d->q; bp.s1_sb = d->q_stride[0]; bp.s1_sh = d->q_stride[1]; bp.s1_sl = d->q_stride[2];
@@ -635,8 +733,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
         bp.out1 = d->dq; bp.o1_sb = d->dq_stride[0]; bp.o1_sh = d->dq_stride[1]; bp.o1_sl = d->dq_stride[2];
         bp.out2 = nullptr; bp.o2_sb = bp.o2_sh = bp.o2_sl = 0;
         bp.stream = k_img; bp.L_stat = d->Lq; bp.L_stream = d->Lkv; bp.n_tiles = g.n_k_tiles;
-        if (!allow_lds((const void*)k_dq, g.lds_dq)) return COSMOS_ATTN_LAUNCH_FAILED;
-        hipLaunchKernelGGL(k_dq, dim3((d->Lq + kBlock - 1) / kBlock, BH), dim3(kBwdThreads), g.lds_dq, stream, bp);
+        if (!launch(k_dq, g.lds_dq, g.dq, bp, false)) return COSMOS_ATTN_LAUNCH_FAILED;
     }
     return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
 }
