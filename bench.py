@@ -1,6 +1,6 @@
 """Benchmark of the attention forward + JVP hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk|dblk] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk|dblk|dblkf] [--no-cpu]
 
 A "step" is one call of the hot path (re-tiling kernel + attention kernel, through the Python host and
 the C ABI) over one batch of synthetic tensors that are already resident in HBM.  Default workload: the
@@ -51,6 +51,7 @@ WORKLOADS = {
     # RMSNorm + RoPE (+ tangent) of q and k, attention forward + JVP
     "blk": ("2B DiT self-attention module fwd+JVP bf16 720p B1 L84480 K2048 H16 d128", 1, 16, 84480, 84480, 128, "module", False, False),
     # one whole DiT block with a tangent: adaLN modulation, self-attention, text cross-attention, MLP, gated residuals
+    "dblkf": ("2B DiT block forward (inference) bf16 720p B1 T24 H44 W80 D2048 heads16 text512x1024 adaLN-LoRA256", 1, 16, 84480, 512, 128, "block_fwd", False, False),
     "dblk": ("2B DiT block fwd+JVP bf16 720p B1 T24 H44 W80 D2048 heads16 text512x1024 adaLN-LoRA256", 1, 16, 84480, 512, 128, "block", False, False),
 }
 PEAK_HBM_GBS = 8000.0
@@ -212,8 +213,9 @@ def bench_module(args, pkg, dev, desc_txt, B, H, L, D):
     print(json.dumps(result), flush=True)
 
 
-def bench_block(args, pkg, dev, desc_txt, B, H, L, Mk, D):
-    """One step = Block.forward_jvp of the 2B DiT's transformer block at the 720p token grid."""
+def bench_block(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False):
+    """One step = Block.forward_jvp (or, with ``forward_only``, Block.forward under no_grad) of the 2B DiT's transformer
+    block at the 720p token grid."""
     nro = entry.load_norm_rope_oracle()
     K, Kc, T, Hh, W = H * D, 1024, 24, 44, 80
     assert T * Hh * W == L
@@ -239,8 +241,17 @@ def bench_block(args, pkg, dev, desc_txt, B, H, L, Mk, D):
         "cross_attn": 4 * 2.0 * B * H * L * Mk * D,
         "mlp": 2 * 2 * gemm(B * L, K, 4 * K),
     }
-    total = sum(flops.values())
     step = lambda: m.forward_jvp(x, tx, emb, temb, ctx, rope, lora, tlora)
+    if forward_only:     # no tangents: half the GEMM work, 2 attention matmuls instead of 6 (4)
+        flops = {k: v / 2 for k, v in flops.items()}
+        flops["self_attn"] = 2 * 2.0 * B * H * L * L * D
+        flops["cross_attn"] = 2 * 2.0 * B * H * L * Mk * D
+        flops["cross_attn_projections"] = 2 * gemm(B * L, K, K) + 2 * gemm(B * Mk, Kc, K)
+
+        def step():
+            with torch.no_grad():
+                return m(x, emb, ctx, rope, lora)
+    total = sum(flops.values())
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -256,7 +267,7 @@ def bench_block(args, pkg, dev, desc_txt, B, H, L, Mk, D):
     del out
     achieved = total / (avg * 1e-3) / 1e12
     result = {
-        "metric": "DiT block fwd+JVP TFLOP/s & % bf16 MFMA peak @ 2B 720p (L=84480); ms per call",
+        "metric": ("DiT block forward" if forward_only else "DiT block fwd+JVP") + " TFLOP/s & % bf16 MFMA peak @ 2B 720p (L=84480); ms per call",
         "value": total / sec / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
@@ -264,7 +275,7 @@ def bench_block(args, pkg, dev, desc_txt, B, H, L, Mk, D):
                    "pct_of_bf16_mfma_peak": 100.0 * total / sec / 1e12 / PEAK_BF16_TFLOPS},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
-                     "kernel": "whole block call (attn_fwd_jvp_kernel dominates)", "kernel_ms_avg": avg},
+                     "kernel": "whole block call (the attention kernel dominates)", "kernel_ms_avg": avg},
     }
     print(json.dumps(result), flush=True)
 
@@ -366,8 +377,8 @@ def main():
     desc_txt, B, H, Lq, Lkv, d, tangents, rms, padded = WORKLOADS[args.workload]
     if tangents == "bwd":
         return bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
-    if tangents == "block":
-        return bench_block(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
+    if tangents in ("block", "block_fwd"):
+        return bench_block(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, forward_only=tangents == "block_fwd")
     if tangents == "module":
         return bench_module(args, pkg, dev, desc_txt, B, H, Lq, d)
     if tangents in ("norm_rope", "norm_rope_bwd"):

@@ -47,7 +47,10 @@ class GPT2FeedForward(nn.Module):
         torch.nn.init.trunc_normal_(self.layer2.weight, std=std, a=-3 * std, b=3 * std)
 
     def forward(self, x: torch.Tensor):
-        return self.layer2(self.activation(self.layer1(x)))
+        h = self.layer1(x)
+        if not torch.is_grad_enabled() and h.is_cuda and h.numel() % 8 == 0:
+            return self.layer2(ops.gelu(h, inplace=True)[0])      # inference: one fused pass, in place
+        return self.layer2(self.activation(h))
 
     @torch.no_grad()
     def forward_jvp(self, x: torch.Tensor, tx: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -175,6 +178,8 @@ class Block(nn.Module):
         if extra_per_block_pos_emb is not None:
             x = x + extra_per_block_pos_emb
         B, T, H, W, D = x.shape
+        if not torch.is_grad_enabled() and x.is_cuda:
+            return self._forward_fused(x, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D, adaln_lora_B_T_3D)
         shift, scale, gate = self._modulation(self.adaln_modulation_self_attn, emb_B_T_D, adaln_lora_B_T_3D, x)
         n = self._modulate(self.layer_norm_self_attn, x, scale, shift)
         r = self.self_attn(n.reshape(B, T * H * W, D), None, rope_emb=rope_emb_L_1_1_D).reshape(B, T, H, W, D)
@@ -186,6 +191,23 @@ class Block(nn.Module):
         shift, scale, gate = self._modulation(self.adaln_modulation_mlp, emb_B_T_D, adaln_lora_B_T_3D, x)
         n = self._modulate(self.layer_norm_mlp, x, scale, shift)
         x = x + gate * self.mlp(n)
+        return x
+
+    def _forward_fused(self, x, emb, crossattn_emb, rope, lora):
+        """Inference (no autograd): the same arithmetic with LayerNorm + modulation, the gated residuals and GELU each as
+        one fused HIP pass instead of a chain of tensor-library ops."""
+        B, T, H, W, D = x.shape
+        flat2 = lambda m: m.reshape(-1, D)
+        for name, norm, sub in (("self_attn", self.layer_norm_self_attn, self.self_attn),
+                                ("cross_attn", self.layer_norm_cross_attn, self.cross_attn),
+                                ("mlp", self.layer_norm_mlp, self.mlp)):
+            shift, scale, gate = self._modulation(getattr(self, "adaln_modulation_" + name), emb, lora, x)
+            n, _ = ops.ln_modulate(x, flat2(shift), flat2(scale), eps=norm.eps)
+            if name == "mlp":
+                r = sub(n)
+            else:
+                r = sub(n.reshape(B, T * H * W, D), None if name == "self_attn" else crossattn_emb, rope_emb=rope)
+            x, _ = ops.gated_residual(x, r.reshape(x.shape), flat2(gate))
         return x
 
     # ------------------------------------------------------------------ forward mode

@@ -105,6 +105,23 @@ def test_block_with_image_context(pkg, oracle, nr_oracle, block_oracle, gpu):
     check(oracle, "out - x", out.float().cpu() - x.float(), want - x.float(), rel_l2=2e-2)
 
 
+def test_inference_path_matches_autograd_path(pkg, oracle, nr_oracle, gpu):
+    """Under no_grad the block runs the fused elementwise passes; with autograd it runs tensor-library ops around the same
+    kernels.  Same arithmetic up to the 16-bit roundings between the unfused ops."""
+    B, T, Hh, W, D, H, Mk, Kc = 1, 2, 4, 8, 256, 2, 24, 96
+    m = build(pkg, gpu, D, Kc, H, 16, torch.bfloat16, 21)
+    g = torch.Generator().manual_seed(22)
+    r = lambda *s: torch.randn(*s, generator=g).bfloat16().to(gpu)
+    x, emb, ctx, lora = r(B, T, Hh, W, D), r(B, T, D), r(B, Mk, Kc), 0.3 * r(B, T, 3 * D)
+    hd = D // H
+    rope = torch.from_numpy(nr_oracle.rope_angles_3d(T, Hh, W, hd)).reshape(-1, 1, 1, hd).to(gpu)
+    with torch.no_grad():
+        fused = m(x, emb, ctx, rope, lora)
+    with torch.enable_grad():
+        plain = m(x.clone().requires_grad_(True), emb, ctx, rope, lora)
+    check(oracle, "fused vs autograd path", fused, plain.detach().float().cpu(), rel_l2=1e-2)
+
+
 def test_fresh_block_is_the_identity(pkg, nr_oracle, gpu):
     """minimal_v4_dit.py:1095-1111: after init_weights the gates are zero."""
     torch.manual_seed(0)
