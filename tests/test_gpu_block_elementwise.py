@@ -125,3 +125,26 @@ def test_gelu_tails(pkg, block_oracle, gpu):
     check("a", a, want, torch.bfloat16)
     check("ta", ta, twant, torch.bfloat16)
     assert torch.isfinite(a.float()).all() and torch.isfinite(ta.float()).all()
+
+
+def test_more_than_2_31_elements(pkg, block_oracle, gpu):
+    """Offsets beyond 32 bits in the three elementwise kernels: 2.4e9-element tensors, checked at both ends."""
+    rows, D, rpg = 1179648, 2048, 4096
+    assert rows * D > 2 ** 31
+    g = torch.Generator(device=gpu).manual_seed(4)
+    x = torch.empty(rows, D, device=gpu, dtype=torch.bfloat16)
+    for i in range(0, rows, 131072):
+        x[i:i + 131072] = torch.randn(131072, D, generator=g, device=gpu).bfloat16()
+    mod = torch.randn(3, rows // rpg, D, generator=g, device=gpu).bfloat16()
+    ends = torch.cat([torch.arange(0, 8), torch.arange(rows - 8, rows)]).to(gpu)
+    grp = (ends // rpg)
+    y, _ = pkg.ln_modulate(x, mod[0], mod[1])
+    want, _ = block_oracle.ln_modulate_torch(x[ends].cpu(), mod[0][grp].cpu(), mod[1][grp].cpu())
+    check("ln_modulate ends", y[ends], want, torch.bfloat16)
+    out, _ = pkg.gated_residual(x, y, mod[2])
+    want, _ = block_oracle.gated_residual_torch(x[ends].cpu(), y[ends].cpu(), mod[2][grp].cpu())
+    check("gated_residual ends", out[ends], want, torch.bfloat16)
+    del out
+    a, _ = pkg.gelu(x)
+    want, _ = block_oracle.gelu_torch(x[ends].cpu())
+    check("gelu ends", a[ends], want, torch.bfloat16)
