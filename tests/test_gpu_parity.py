@@ -394,6 +394,35 @@ def sampled_rows_check(pkg, oracle, gpu, H, Lq, Lkv, tangents, rms, key_lens=Non
     return (q, k, v, tq, tk, tv), (o, to, lse)
 
 
+def test_more_than_2_31_elements(pkg, oracle, gpu):
+    """Offsets beyond 32 bits: q, k, v and tangents of 2.2e9 elements each (B=4, H=128, L=32896, d=128), generated on the
+    GPU; row blocks of the first and of the last (batch, head) against the row-block oracle, forward + JVP and forward only."""
+    B, H, L, d = 4, 128, 32896, 128
+    assert B * H * L * d > 2 ** 31
+    g = torch.Generator(device=gpu).manual_seed(0)
+
+    def rn(std):
+        x = torch.empty(B, H, L, d, device=gpu, dtype=torch.bfloat16)
+        for b in range(B):
+            x[b] = (torch.randn(H, L, d, generator=g, device=gpu) * std).bfloat16()
+        return x
+
+    q, k, v, tq, tk, tv = rn(1.0), rn(1.0), rn(1.0), rn(0.1), rn(0.1), rn(0.1)
+    o, to, lse = pkg.fwd_jvp(q, k, v, tq, tk, tv)
+    o_f, _, lse_f = pkg.fwd_jvp(q, k, v)
+    torch.cuda.synchronize()
+    c = lambda x: x.cpu()
+    for b, h, r0 in ((0, 0, 0), (B - 1, H - 1, 0), (B - 1, H - 1, L - 128), (2, 77, 12345)):
+        rows = slice(r0, r0 + 128)
+        o_ref, to_ref, lse_ref = oracle.rows_oracle(c(q[b, h, rows]), c(k[b, h]), c(v[b, h]), c(tq[b, h, rows]), c(tk[b, h]), c(tv[b, h]))
+        print(f" rows {r0}..{r0 + 128} of (b={b}, h={h})", flush=True)
+        check(oracle, "o", o[b, h, rows], o_ref)
+        check(oracle, "to", to[b, h, rows], to_ref)
+        check(oracle, "o (forward only)", o_f[b, h, rows], o_ref)
+        assert oracle.error_metrics(lse[b, h, rows].cpu(), lse_ref)[0] <= LSE_ABS
+        assert oracle.error_metrics(lse_f[b, h, rows].cpu(), lse_ref)[0] <= LSE_ABS
+
+
 def test_config3_shape_2b_720p_fwd_jvp(pkg, oracle, gpu):
     """The 2B 720p forward + JVP configuration at its real sequence length (L=84480, d=128, bf16, primals N(0,1), tangents N(0,1)*0.1) on 2 of
     the 16 heads (heads are independent; the full-H run is bench.py's), plus properties that need no oracle."""
