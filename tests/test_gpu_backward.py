@@ -151,6 +151,24 @@ def test_bwd_config3_shape_sampled(pkg, oracle, gpu):
         check(oracle, f"dq rows {r0}", dq[:, :, r0:r0 + 128], ref.double().numpy())
 
 
+@pytest.mark.parametrize("chunk", range(2))
+def test_bwd_random_shapes(pkg, oracle, gpu, chunk):
+    """16 seeded random cases: batch, heads, lengths, head dim, dtype, causal drawn at random (workgroup counts on either
+    side of the thresholds at which the last round is cut along the stream)."""
+    import numpy as np
+
+    rng = np.random.default_rng(2000 + chunk)
+    for _ in range(8):
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 13))
+        Lq, Lkv = int(rng.integers(1, 900)), int(rng.integers(1, 1200))
+        d = int(rng.choice([16, 32, 64, 128]))
+        causal = rng.random() < 0.2
+        if causal:
+            Lkv = Lq
+        dtype = torch.float16 if rng.random() < 0.3 else torch.bfloat16
+        run_bwd(pkg, oracle, gpu, (B, H, Lq, d), (B, H, Lkv, d), causal=causal, seed=int(rng.integers(0, 10000)), dtype=dtype)
+
+
 def test_bwd_more_than_2_31_elements(pkg, oracle, gpu):
     """Offsets beyond 32 bits in the backward: tensors of 2.2e9 elements (B=4, H=128, L=32896, d=128) generated on the
     GPU; the last (batch, head) against the closed-form oracle restricted to that head (heads are independent)."""

@@ -144,6 +144,29 @@ def test_forward_only_key_range_split(pkg, oracle, gpu, shape_q, Lkv, ranges):
     assert torch.equal(o_again, o_ref) and torch.equal(lse_again, lse_ref)
 
 
+@pytest.mark.parametrize("chunk", range(4))
+def test_random_shapes_all_modes(pkg, oracle, gpu, chunk):
+    """40 seeded random cases (10 per chunk): batch, heads, lengths, head dims, dtype and tangent set drawn at random --
+    workgroup counts on either side of the thresholds at which the last round is cut along the keys, key-tile counts
+    around the ring depths, ragged ends."""
+    rng = np.random.default_rng(1000 + chunk)
+    for _ in range(10):
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 13))
+        Lq, Lkv = int(rng.integers(1, 1000)), int(rng.integers(1, 1600))
+        d = int(rng.choice([16, 32, 64, 128]))
+        dv = int(rng.choice([16, 32, 64, 128])) if rng.random() < 0.3 else d
+        tangents = str(rng.choice(["full", "q", "none", "kv"]))
+        dtype = torch.float16 if rng.random() < 0.3 else torch.bfloat16
+        mask = rng.random()
+        causal, key_lens = False, None
+        if mask < 0.15:
+            causal, Lkv = True, Lq
+        elif mask < 0.3:
+            key_lens = [int(x) for x in rng.integers(1, Lkv + 1, B)]
+        run_case(pkg, oracle, gpu, (B, H, Lq, d), (B, H, Lkv, d), dv=dv, causal=causal, key_lens=key_lens,
+                 seed=int(rng.integers(0, 10000)), dtype=dtype, tangents=tangents)
+
+
 def test_against_torch_sdpa_jvp(pkg, oracle, gpu):
     """The quoted oracle itself (torch math SDPA under torch.func.jvp, fp32) on a mid-size case."""
     q, k, v, tq, tk, tv = oracle.make_inputs((2, 3, 300, 128), seed=5)
