@@ -371,6 +371,34 @@ def test_hip_graph_capture_and_replay(pkg, oracle, gpu):
         assert torch.equal(o_g, o_e) and torch.equal(to_g, to_e) and torch.equal(lse_g, lse_e), seed
 
 
+def test_hip_graph_capture_with_key_range_split(pkg, oracle, gpu):
+    """The cut of a thin last round (several launches: attention kernel + merge kernel, scratch in the caller's workspace)
+    under graph capture: replays match eager calls bit for bit, forward only and forward + JVP."""
+    make = lambda seed: [x.to(gpu) for x in oracle.make_inputs((1, 2, 1000, 128), (1, 2, 1000, 128), seed=seed)]
+    static = make(0)
+    pkg.fwd_jvp(*static); pkg.fwd_jvp(*static[:3])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        pkg.fwd_jvp(*static); pkg.fwd_jvp(*static[:3])
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o_g, to_g, lse_g = pkg.fwd_jvp(*static)
+        of_g, _, lsef_g = pkg.fwd_jvp(*static[:3])
+    for seed in (1, 2):
+        fresh = make(seed)
+        for dst, src in zip(static, fresh):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        o_e, to_e, lse_e = pkg.fwd_jvp(*fresh)
+        of_e, _, lsef_e = pkg.fwd_jvp(*fresh[:3])
+        torch.cuda.synchronize()
+        assert torch.equal(o_g, o_e) and torch.equal(to_g, to_e) and torch.equal(lse_g, lse_e), seed
+        assert torch.equal(of_g, of_e) and torch.equal(lsef_g, lsef_e), seed
+
+
 def test_golden_fixtures(pkg, oracle, gpu):
     spec = importlib.util.spec_from_file_location("make_golden", os.path.join(GOLDEN_DIR, "make_golden.py"))
     mg = importlib.util.module_from_spec(spec)
