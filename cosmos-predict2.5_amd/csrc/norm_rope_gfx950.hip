@@ -352,7 +352,7 @@ __global__ void __launch_bounds__(kThreads) norm_rope_dweight_kernel(const float
     red[threadIdx.x] = t;
     __syncthreads();
     for (int w = kThreads / 2; w > 0; w >>= 1) {
-        if (threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
         __syncthreads();
     }
     if (threadIdx.x == 0) dweight[j] = red[0];
