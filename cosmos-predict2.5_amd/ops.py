@@ -95,15 +95,15 @@ def fwd_jvp(
 
     if out_layout == "bhld":
         o = torch.empty((B, H, Lq, d_v), device=q.device, dtype=q.dtype)
-    elif out_layout == "blhd":
-        o = torch.empty((B, Lq, H, d_v), device=q.device, dtype=q.dtype).transpose(1, 2)
-    else:
-        raise ValueError(f"out_layout={out_layout!r}")
-    to = torch.empty_like(o) if have_tangent else None  # empty_like keeps o's strides
-    if have_tangent and out_layout == "blhd":
+        to = torch.empty_like(o) if have_tangent else None
+    elif out_layout == "blhd" and have_tangent:
         # o and to as the two halves of one buffer: a following linear layer maps both in one GEMM without a copy
         both = torch.empty((2, B, Lq, H, d_v), device=q.device, dtype=q.dtype)
         o, to = both[0].transpose(1, 2), both[1].transpose(1, 2)
+    elif out_layout == "blhd":
+        o, to = torch.empty((B, Lq, H, d_v), device=q.device, dtype=q.dtype).transpose(1, 2), None
+    else:
+        raise ValueError(f"out_layout={out_layout!r}")
     lse = torch.empty((B, H, Lq), device=q.device, dtype=torch.float32) if need_lse else None
 
     if key_lens is not None:
