@@ -605,19 +605,14 @@ struct BwdGeom {
         const size_t p2 = (size_t)dq.n_rem * dq.splits * kBlock * d->d * sizeof(float);
         part_bytes = ((p1 > p2 ? p1 : p2) + 1023) / 1024 * 1024;     // the two kernels run one after the other
     }
-    // How the (block of stationary rows, head) pairs of a kernel are dealt out.  One workgroup fits on a compute unit, so
-    // a launch runs in rounds of kNumCUs; when the last round is less than half full its pairs are cut along the stream
-    // into as many ranges as fill it, and bwd_combine_kernel adds the ranges up.
+    // How the (block of stationary rows, head) pairs of a kernel are dealt out (see choose_splits): the pairs of a partly
+    // filled last round of workgroups are cut along the stream and bwd_combine_kernel adds the ranges up.
     struct Plan { int n_blk, n_pairs, n_full, n_rem, splits; };
     static Plan plan(int n_blk, int bh, int n_stream_tiles, bool causal) {
-        constexpr int kNumCUs = 256, kMaxSplits = 16, kMinStepsPerSplit = 4;
         Plan s;
         s.n_blk = n_blk; s.n_pairs = n_blk * bh; s.n_full = s.n_pairs; s.n_rem = 0; s.splits = 1;
         const int rem = s.n_pairs % kNumCUs;
-        if (causal || rem == 0 || rem > kNumCUs / 2) return s;
-        int splits = kNumCUs / rem;
-        if (splits > kMaxSplits) splits = kMaxSplits;
-        if (splits > n_stream_tiles / kMinStepsPerSplit) splits = n_stream_tiles / kMinStepsPerSplit;
+        const int splits = causal ? 1 : choose_splits(rem, n_stream_tiles);
         if (splits < 2) return s;
         s.n_rem = rem; s.n_full = s.n_pairs - rem; s.splits = splits;
         return s;

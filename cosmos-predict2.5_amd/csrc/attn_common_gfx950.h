@@ -73,6 +73,25 @@ inline bool allow_lds(const void* fn, size_t bytes) {
     return true;
 }
 
+// One workgroup of the attention kernels fits on a compute unit, so a launch of n_pairs equal workgroups runs in rounds
+// of kNumCUs and a partly filled last round costs a whole one.  The `rem` workgroups of that round may instead be cut
+// into S ranges of their stream (keys or queries) each: rem * S shorter workgroups that take ceil(rem S / kNumCUs) / S
+// of a round, plus a merge kernel.  Returns the smallest S (1 = leave it) that minimises that cost, among the S that
+// leave every range at least kMinStepsPerSplit barrier steps, if it saves at least a tenth of a round.
+constexpr int kNumCUs = 256;          // MI355X
+constexpr int kMaxSplits = 16;
+constexpr int kMinStepsPerSplit = 4;
+inline int choose_splits(int rem, int n_steps) {
+    if (rem <= 0) return 1;
+    int best = 1;
+    double best_cost = 1.0;
+    for (int S = 2; S <= kMaxSplits && S * kMinStepsPerSplit <= n_steps; ++S) {
+        const double cost = (double)((rem * S + kNumCUs - 1) / kNumCUs) / S;
+        if (cost < best_cost - 1e-9) { best_cost = cost; best = S; }
+    }
+    return best_cost <= 0.9 ? best : 1;
+}
+
 inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 inline bool strides_ok(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0; }
 inline bool head_dim_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }

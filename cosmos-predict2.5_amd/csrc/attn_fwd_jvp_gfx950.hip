@@ -989,12 +989,8 @@ int n_tiles_of(const cosmos_attn_desc* d) { return (d->Lkv + kBlockN - 1) / kBlo
 // workspace = packed tiles [B*H][n_tiles][tile bytes]
 size_t tiles_bytes_of(const cosmos_attn_desc* d) { return (size_t)d->B * d->H * n_tiles_of(d) * tile_bytes_of(d); }
 
-// How the (query block, head) pairs are dealt out.  One workgroup fits on a compute unit, so a launch runs in rounds of
-// kNumCUs workgroups; when the last round is less than half full its pairs are cut along the keys into as many ranges
-// as fill it, and a small second kernel merges the ranges.
-constexpr int kNumCUs = 256;
-constexpr int kMaxSplits = 16;
-constexpr int kMinStepsPerSplit = 4;      // in barrier steps: 64 keys forward only, 32 keys with tangents
+// How the (query block, head) pairs are dealt out (see choose_splits): the pairs of a partly filled last round of
+// workgroups are cut along the keys, and a small second kernel merges the ranges.
 struct SplitPlan { int block_m, n_qt, n_pairs, n_full, n_rem, splits; };
 SplitPlan plan_split(const cosmos_attn_desc* d) {
     SplitPlan s;
@@ -1005,11 +1001,8 @@ SplitPlan plan_split(const cosmos_attn_desc* d) {
     s.n_rem = 0; s.splits = 1; s.n_full = s.n_pairs;
     if (d->causal || d->key_lens) return s;          // key ranges of equal work only
     const int rem = s.n_pairs % kNumCUs;
-    const int n_steps = fwd ? (n_tiles_of(d) + 1) / 2 : n_tiles_of(d);
-    if (rem == 0 || rem > kNumCUs / 2) return s;
-    int splits = kNumCUs / rem;
-    if (splits > kMaxSplits) splits = kMaxSplits;
-    if (splits > n_steps / kMinStepsPerSplit) splits = n_steps / kMinStepsPerSplit;
+    const int n_steps = fwd ? (n_tiles_of(d) + 1) / 2 : n_tiles_of(d);   // barrier steps: 64 keys forward only, 32 with tangents
+    const int splits = choose_splits(rem, n_steps);
     if (splits < 2) return s;
     s.n_rem = rem; s.n_full = s.n_pairs - rem; s.splits = splits;
     return s;
