@@ -24,32 +24,18 @@ from __future__ import annotations
 from typing import Dict, Optional
 
 
-def block_torch(weights: Dict[str, "torch.Tensor"], x, emb, crossattn_emb, rope_angles=None, num_heads: int = 8,
-                adaln_lora=None, tx=None, temb=None, tadaln_lora=None, dtype=None, keep_graph_input=None):
-    """weights: the block's state dict.  x: [B, T, H, W, D]; emb: [B, T, D]; crossattn_emb: [B, Mk, Kc], or the pair
-    (text context, image context [B, Mi, Ki]) when the state dict holds the image-conditioned cross-attention
-    (``cross_attn.k_img.weight`` ...: minimal_v4_dit.py:451-493, the two attention results are summed before the output
-    projection);
-    rope_angles: [T*H*W, D/num_heads] or None; adaln_lora: [B, T, 3 D] (required iff the state dict holds the
-    LoRA form of the modulation).  Returns (out, tout); tout is None without tx."""
+def make_block_forward(w, num_heads: int, rope_angles, ctx, img_ctx=None):
+    """The block as a pure function ``fwd(x [B,T,H,W,D], emb [B,T,D], adaln_lora [B,T,3D] or 0-d) -> [B,T,H,W,D]`` of
+    torch tensors that already sit on the CPU in one dtype (w: state dict; rope_angles: [T*H*W, head_dim] or None;
+    ctx: text context; img_ctx: image context or None)."""
     import torch
     import torch.nn.functional as F
     from torch.nn.attention import SDPBackend, sdpa_kernel
 
-    dt = dtype or torch.float32
-    f = lambda t: None if t is None else torch.as_tensor(t).detach().to("cpu", dt)
-    w = {k: f(v) for k, v in weights.items()}
-    img_ctx = None
-    if isinstance(crossattn_emb, (tuple, list)):
-        crossattn_emb, img_ctx = crossattn_emb
-        img_ctx = f(img_ctx)
-    x, emb, ctx, lora, tx, temb, tlora = (f(t) for t in (x, emb, crossattn_emb, adaln_lora, tx, temb, tadaln_lora))
-    if keep_graph_input is not None:
-        x = keep_graph_input.to(dt)
-    B, T, H, W, D = x.shape
-    hd = D // num_heads
-    a = None if rope_angles is None else f(rope_angles).reshape(1, -1, 1, hd)
     use_lora = "adaln_modulation_mlp.2.weight" in w
+    D = w["mlp.layer2.weight"].shape[0]
+    hd = D // num_heads
+    a = None if rope_angles is None else rope_angles.reshape(1, -1, 1, hd)
 
     def modulation(name, e, l):
         m = F.linear(F.silu(e), w[f"adaln_modulation_{name}.1.weight"])
@@ -77,6 +63,7 @@ def block_torch(weights: Dict[str, "torch.Tensor"], x, emb, crossattn_emb, rope_
         return F.linear(o.flatten(-2), w[prefix + "output_proj.weight"])
 
     def fwd(x_, e_, l_):
+        B, T, H, W, _ = x_.shape
         ln = lambda t: F.layer_norm(t, (D,), eps=1e-6)
         shift, scale, gate = modulation("self_attn", e_, l_)
         n = (ln(x_) * (1 + scale) + shift).reshape(B, T * H * W, D)
@@ -87,6 +74,32 @@ def block_torch(weights: Dict[str, "torch.Tensor"], x, emb, crossattn_emb, rope_
         shift, scale, gate = modulation("mlp", e_, l_)
         n = ln(x_) * (1 + scale) + shift
         return x_ + gate * F.linear(F.gelu(F.linear(n, w["mlp.layer1.weight"])), w["mlp.layer2.weight"])
+
+    return fwd
+
+
+def block_torch(weights: Dict[str, "torch.Tensor"], x, emb, crossattn_emb, rope_angles=None, num_heads: int = 8,
+                adaln_lora=None, tx=None, temb=None, tadaln_lora=None, dtype=None, keep_graph_input=None):
+    """weights: the block's state dict.  x: [B, T, H, W, D]; emb: [B, T, D]; crossattn_emb: [B, Mk, Kc], or the pair
+    (text context, image context [B, Mi, Ki]) when the state dict holds the image-conditioned cross-attention
+    (``cross_attn.k_img.weight`` ...: minimal_v4_dit.py:451-493, the two attention results are summed before the output
+    projection);
+    rope_angles: [T*H*W, D/num_heads] or None; adaln_lora: [B, T, 3 D] (required iff the state dict holds the
+    LoRA form of the modulation).  Returns (out, tout); tout is None without tx."""
+    import torch
+
+    dt = dtype or torch.float32
+    f = lambda t: None if t is None else torch.as_tensor(t).detach().to("cpu", dt)
+    w = {k: f(v) for k, v in weights.items()}
+    img_ctx = None
+    if isinstance(crossattn_emb, (tuple, list)):
+        crossattn_emb, img_ctx = crossattn_emb
+        img_ctx = f(img_ctx)
+    x, emb, ctx, lora, tx, temb, tlora = (f(t) for t in (x, emb, crossattn_emb, adaln_lora, tx, temb, tadaln_lora))
+    if keep_graph_input is not None:
+        x = keep_graph_input.to(dt)
+    a = None if rope_angles is None else f(rope_angles)
+    fwd = make_block_forward(w, num_heads, a, ctx, img_ctx)
 
     if lora is None:
         lora = torch.zeros((), dtype=dt)

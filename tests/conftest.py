@@ -35,6 +35,11 @@ def block_oracle():
 
 
 @pytest.fixture(scope="session")
+def net_oracle():
+    return entry.load_dit_network_oracle()
+
+
+@pytest.fixture(scope="session")
 def pkg():
     """The package with its HIP library loaded; fails loudly when the library is not built."""
     return entry.load_package()

@@ -1,0 +1,143 @@
+"""GPU parity of the DiT network (patch embedding, time embedding, blocks on the HIP kernels, final layer, unpatchify)
+and of its forward-mode tangent along (x, timesteps) against the CPU oracle of the network (torch fp32 under
+torch.func.jvp, pinned in tests/test_oracle_dit_network.py) on the same 16-bit weights and inputs.
+
+Tolerance: the output is ``linear(layer_norm(...))`` of a stream that went through every block in 16 bits, with no
+residual carrying it: relative-L2 <= 2e-2 and max-abs <= 5e-2 * max(1, max|want|), for output and tangent alike.
+"""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def check(oracle, name, got, want, rel_l2=2e-2, max_abs=5e-2):
+    ma, rl = oracle.error_metrics(got.float().cpu(), want)
+    lim = max_abs * max(1.0, float(want.abs().max()))
+    print(f"  {name}: max_abs={ma:.3e} (limit {lim:.3e}) rel_l2={rl:.3e}", flush=True)
+    assert math.isfinite(ma) and ma <= lim, f"{name}: max-abs {ma} > {lim}"
+    assert rl <= rel_l2, f"{name}: rel-L2 {rl} > {rel_l2}"
+
+
+def build(pkg, gpu, dtype, seed, **kw):
+    torch.manual_seed(seed)
+    net = pkg.MiniTrainDIT(**kw)
+    with torch.no_grad():    # the reference starts every last modulation layer at zero: make them do something
+        for blk in net.blocks:
+            for mod in (blk.adaln_modulation_self_attn, blk.adaln_modulation_cross_attn, blk.adaln_modulation_mlp):
+                mod[-1].weight.copy_(torch.randn_like(mod[-1].weight) / mod[-1].weight.shape[1] ** 0.5)
+            for att in (blk.self_attn, blk.cross_attn):
+                att.q_norm.weight.add_(0.2 * torch.randn_like(att.q_norm.weight))
+                att.k_norm.weight.add_(0.2 * torch.randn_like(att.k_norm.weight))
+        last = net.final_layer.adaln_modulation[-1].weight
+        last.copy_(torch.randn_like(last) / last.shape[1] ** 0.5)
+        net.t_embedding_norm.weight.add_(0.2 * torch.randn_like(net.t_embedding_norm.weight))
+    return net.to(device=gpu, dtype=dtype).eval()
+
+
+def run(pkg, oracle, net_oracle, gpu, *, B, C, T, Hh, W, Mk, Kin, dtype=torch.bfloat16, seed=0, per_frame_time=False, img=None, **kw):
+    print(f"network case B={B} C={C} T={T} H={Hh} W={W} Mk={Mk} {dtype} seed={seed} {kw}", flush=True)
+    net = build(pkg, gpu, dtype, seed, in_channels=C, **kw)
+    p, r, heads = kw["patch_spatial"], kw["patch_temporal"], kw["num_heads"]
+    g = torch.Generator().manual_seed(seed + 1)
+    rn = lambda *s: torch.randn(*s, generator=g)
+    x, tx = rn(B, C, T, Hh, W).to(dtype), (0.3 * rn(B, C, T, Hh, W)).to(dtype)
+    Tt = T // r if per_frame_time else 1
+    ts = (torch.rand(B, Tt, generator=g) * 1.4 + 0.05).to(dtype)
+    tts = (0.2 * rn(B, Tt)).to(dtype)
+    ctx = rn(B, Mk, Kin).to(dtype)
+    imgc = None if img is None else rn(B, *img).to(dtype)
+    pm = (torch.rand(B, 1, Hh, W, generator=g) > 0.5).to(dtype) if kw.get("concat_padding_mask", True) else None
+    fps = torch.full((B,), 16.0)
+    d = lambda t: None if t is None else t.to(gpu)
+    with torch.no_grad():
+        out = net(d(x), d(ts), d(ctx), fps=d(fps), padding_mask=d(pm), img_context_emb=d(imgc))
+    out2, tout = net.forward_jvp(d(x), d(tx), d(ts), d(tts), d(ctx), fps=d(fps), padding_mask=d(pm), img_context_emb=d(imgc))
+    torch.cuda.synchronize()
+    assert out.shape == (B, kw["out_channels"], T, Hh, W) and out.dtype == dtype and tout.shape == out.shape
+    with torch.no_grad():
+        angles = net.pos_embedder.generate_embeddings((B, T // r, Hh // p, W // p, 0), fps=d(fps)).reshape(-1, kw["model_channels"] // heads)
+    want, twant = net_oracle.network_torch(net.state_dict(), x, ts, ctx, num_heads=heads, patch_spatial=p, patch_temporal=r,
+                                           rope_angles=angles.cpu(), padding_mask=pm, img_context_emb=imgc, tx=tx, ttimesteps=tts)
+    check(oracle, "out", out, want)
+    check(oracle, "out (jvp call)", out2, want)
+    check(oracle, "tout", tout, twant)
+    return net, (x, tx, ts, tts, ctx, pm, fps)
+
+
+SMALL = dict(max_img_h=32, max_img_w=32, max_frames=8, out_channels=4, patch_spatial=2, patch_temporal=1, model_channels=256,
+             num_blocks=2, num_heads=2, crossattn_emb_channels=96)
+
+
+@pytest.mark.parametrize("lora_dim", [0, 16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_network_small(pkg, oracle, net_oracle, gpu, lora_dim, dtype):
+    run(pkg, oracle, net_oracle, gpu, B=2, C=4, T=2, Hh=8, W=12, Mk=20, Kin=96, dtype=dtype, seed=lora_dim,
+        use_adaln_lora=bool(lora_dim), adaln_lora_dim=lora_dim or 256, **SMALL)
+
+
+def test_network_all_options(pkg, oracle, net_oracle, gpu):
+    """Per-frame timesteps, learned per-block position term, text-context projection, image context, temporal patches,
+    no padding-mask channel."""
+    kw = dict(SMALL, patch_temporal=2, extra_per_block_abs_pos_emb=True, use_crossattn_projection=True, crossattn_proj_in_channels=80,
+              extra_image_context_dim=48, concat_padding_mask=False, use_adaln_lora=True, adaln_lora_dim=16)
+    run(pkg, oracle, net_oracle, gpu, B=1, C=3, T=4, Hh=8, W=8, Mk=20, Kin=80, seed=5, per_frame_time=True, img=(12, 48), **kw)
+
+
+def test_network_2b_widths_reduced(pkg, oracle, net_oracle, gpu):
+    """The 2B DiT's widths (2048 channels, 16 heads of 128, adaLN-LoRA 256, 16 latent channels in and out, 2 x 2 x 1
+    patches, text context 1024 wide) with 2 blocks on a 3 x 8 x 16 token grid."""
+    kw = dict(max_img_h=240, max_img_w=240, max_frames=128, out_channels=16, patch_spatial=2, patch_temporal=1, model_channels=2048,
+              num_blocks=2, num_heads=16, crossattn_emb_channels=1024, use_adaln_lora=True, adaln_lora_dim=256)
+    run(pkg, oracle, net_oracle, gpu, B=1, C=16, T=3, Hh=16, W=32, Mk=512, Kin=1024, seed=9, **kw)
+
+
+def test_tangent_is_linear_in_its_direction_and_time_direction_matters(pkg, oracle, net_oracle, gpu):
+    net, (x, tx, ts, tts, ctx, pm, fps) = run(pkg, oracle, net_oracle, gpu, B=1, C=4, T=2, Hh=8, W=8, Mk=20, Kin=96, seed=13,
+                                              use_adaln_lora=True, adaln_lora_dim=16, **SMALL)
+    d = lambda t: t.to(gpu)
+    _, t_x = net.forward_jvp(d(x), d(tx), d(ts), None, d(ctx), fps=d(fps), padding_mask=d(pm))
+    _, t_t = net.forward_jvp(d(x), torch.zeros_like(d(tx)), d(ts), d(tts), d(ctx), fps=d(fps), padding_mask=d(pm))
+    _, t_both = net.forward_jvp(d(x), d(tx), d(ts), d(tts), d(ctx), fps=d(fps), padding_mask=d(pm))
+    assert float(t_t.float().abs().max()) > 1e-3
+    check(oracle, "t(x dir) + t(time dir) vs t(both)", t_x.float() + t_t.float(), t_both.float().cpu())
+
+
+def test_inference_path_matches_autograd_path_and_backward_runs(pkg, oracle, net_oracle, gpu):
+    net = build(pkg, gpu, torch.bfloat16, 17, in_channels=4, use_adaln_lora=True, adaln_lora_dim=16, **SMALL).train()
+    g = torch.Generator().manual_seed(18)
+    rn = lambda *s: torch.randn(*s, generator=g).bfloat16().to(gpu)
+    x, ctx = rn(1, 4, 2, 8, 8), rn(1, 20, 96)
+    ts = torch.tensor([[0.7]], device=gpu, dtype=torch.bfloat16)
+    pm = torch.zeros(1, 1, 8, 8, device=gpu, dtype=torch.bfloat16)
+    fps = torch.full((1,), 16.0, device=gpu)
+    with torch.no_grad():
+        fused = net(x, ts, ctx, fps=fps, padding_mask=pm)
+    xg = x.clone().requires_grad_(True)
+    plain = net(xg, ts, ctx, fps=fps, padding_mask=pm)
+    check(oracle, "fused vs autograd path", fused, plain.detach().float().cpu())
+    plain.backward(torch.randn_like(plain))
+    torch.cuda.synchronize()
+    assert torch.isfinite(xg.grad.float()).all() and float(xg.grad.float().abs().max()) > 0
+    for name, prm in net.named_parameters():
+        assert prm.grad is not None and torch.isfinite(prm.grad.float()).all(), name
+
+
+def test_fresh_network_output_does_not_depend_on_time(pkg, gpu):
+    """After init_weights every modulation layer is zero; without adaLN-LoRA the blocks are then the identity, the output is
+    ``linear(layer_norm(x))`` whatever the time, and the tangent along the time is exactly zero."""
+    torch.manual_seed(0)
+    net = pkg.MiniTrainDIT(in_channels=4, use_adaln_lora=False, **SMALL).to(device=gpu, dtype=torch.bfloat16).eval()
+    x = torch.randn(1, 4, 2, 8, 8, device=gpu, dtype=torch.bfloat16)
+    ctx = torch.randn(1, 20, 96, device=gpu, dtype=torch.bfloat16)
+    pm = torch.zeros(1, 1, 8, 8, device=gpu, dtype=torch.bfloat16)
+    fps = torch.full((1,), 16.0, device=gpu)
+    ts = torch.tensor([[0.3]], device=gpu, dtype=torch.bfloat16)
+    out, tout = net.forward_jvp(x, torch.zeros_like(x), ts, torch.ones_like(ts), ctx, fps=fps, padding_mask=pm)
+    with torch.no_grad():
+        a = net(x, ts, ctx, fps=fps, padding_mask=pm)
+        b = net(x, 3 * ts, ctx, fps=fps, padding_mask=pm)
+    assert torch.equal(out, a) and torch.equal(a, b)
+    assert float(tout.float().abs().max()) == 0.0

@@ -321,6 +321,59 @@ def test_dit_block_mirrors_reference_surface(pkg):
         pkg.Block(64, 48, 2, use_wan_fp32_strategy=True)
 
 
+def test_dit_network_mirrors_reference_surface(pkg):
+    """State-dict names of the reference's network (minimal_v4_dit.py:1338-1432) and its host-side pieces, on the CPU."""
+    import numpy as np
+    from einops import rearrange
+
+    net = pkg.MiniTrainDIT(max_img_h=16, max_img_w=16, max_frames=8, in_channels=3, out_channels=5, patch_spatial=2, patch_temporal=1,
+                           model_channels=64, num_blocks=2, num_heads=2, crossattn_emb_channels=48, use_adaln_lora=True, adaln_lora_dim=8,
+                           extra_per_block_abs_pos_emb=True, use_crossattn_projection=True, crossattn_proj_in_channels=40,
+                           extra_image_context_dim=24)
+    keys = set(net.state_dict())
+    for k in ("x_embedder.proj.1.weight", "pos_embedder.seq", "pos_embedder.dim_spatial_range", "pos_embedder.dim_temporal_range",
+              "extra_pos_embedder.pos_emb_h", "extra_pos_embedder.pos_emb_w", "extra_pos_embedder.pos_emb_t",
+              "t_embedder.1.linear_1.weight", "t_embedder.1.linear_2.weight", "t_embedding_norm.weight",
+              "blocks.0.self_attn.q_proj.weight", "blocks.1.cross_attn.k_img_norm.weight", "blocks.1.adaln_modulation_mlp.2.weight",
+              "final_layer.linear.weight", "final_layer.adaln_modulation.1.weight", "final_layer.adaln_modulation.2.weight",
+              "crossattn_proj.0.weight", "crossattn_proj.0.bias", "img_context_proj.0.weight", "img_context_proj.0.bias"):
+        assert k in keys, k
+    assert "t_embedder.1.linear_1.bias" not in keys                      # bias only without adaLN-LoRA (:755)
+    assert net.x_embedder.proj[1].weight.shape == (64, (3 + 1) * 2 * 2 * 1)    # one more channel for the padding mask
+    assert net.t_embedder[1].linear_2.weight.shape == (3 * 64, 64)
+    assert net.final_layer.linear.weight.shape == (2 * 2 * 1 * 5, 64)
+    assert net.blocks[0].cross_attn.k_img.weight.shape == (64, 64)       # image context is projected to model_channels first
+    assert float(net.final_layer.adaln_modulation[2].weight.detach().abs().max()) == 0.0   # init_weights: modulation starts at zero
+    plain = pkg.MiniTrainDIT(max_img_h=16, max_img_w=16, max_frames=8, in_channels=3, out_channels=3, patch_spatial=2, patch_temporal=1,
+                             model_channels=64, num_blocks=1, num_heads=2, concat_padding_mask=False)
+    assert "t_embedder.1.linear_1.bias" in plain.state_dict() and "final_layer.adaln_modulation.2.weight" not in plain.state_dict()
+    for kw in (dict(n_dense_blocks=2), dict(use_wan_fp32_strategy=True), dict(natten_parameters={})):
+        with pytest.raises(NotImplementedError):
+            pkg.MiniTrainDIT(16, 16, 8, 3, 3, 2, 1, model_channels=64, num_blocks=1, num_heads=2, **kw)
+
+    # host-side pieces against einops with the reference's pattern strings / explicit numpy
+    x = torch.randn(2, 4, 4, 6, 8)
+    pe = pkg.PatchEmbed(2, 2, in_channels=4, out_channels=16)
+    want = rearrange(x, "b c (t r) (h m) (w n) -> b t h w (c r m n)", r=2, m=2, n=2) @ pe.proj[1].weight.T
+    assert torch.allclose(pe(x), want, atol=1e-6)
+    y = torch.randn(2, 3, 4, 4, 2 * 2 * 1 * 5)
+    assert torch.equal(net.unpatchify(y), rearrange(y, "B T H W (p1 p2 t C) -> B C (T t) (H p1) (W p2)", p1=2, p2=2, t=1))
+    ts = torch.tensor([[0.5, 2.0], [7.0, 0.1]])
+    ang = ts.numpy()[..., None].astype(np.float64) * 10000.0 ** (-np.arange(32) / 32)
+    assert np.allclose(pkg.Timesteps(64)(ts).numpy(), np.concatenate([np.cos(ang), np.sin(ang)], -1), atol=1e-5)
+    emb, lora = net.t_embedder(ts)
+    assert emb.shape == (2, 2, 64) and lora.shape == (2, 2, 192) and torch.equal(emb, pkg.Timesteps(64)(ts))
+    e = net.extra_pos_embedder(torch.zeros(2, 3, 4, 5, 64))
+    raw = (net.extra_pos_embedder.pos_emb_t[:3, None, None] + net.extra_pos_embedder.pos_emb_h[None, :4, None]
+           + net.extra_pos_embedder.pos_emb_w[None, None, :5]).detach().double().numpy()
+    want = raw / (1e-6 + np.sqrt((raw ** 2).sum(-1, keepdims=True)) / 8.0)
+    assert e.shape == (2, 3, 4, 5, 64) and np.allclose(e[1].detach().numpy(), want, atol=1e-5)
+    pm = torch.zeros(2, 1, 4, 4)
+    pm[:, :, :2] = 1
+    xin = net._with_padding_mask(torch.zeros(2, 3, 2, 8, 8), pm)
+    assert xin.shape == (2, 4, 2, 8, 8) and float(xin[:, 3, :, :4].min()) == 1.0 and float(xin[:, 3, :, 4:].max()) == 0.0
+
+
 def test_rope_position_table_mirrors_reference(pkg, nr_oracle):
     """VideoRopePosition3DEmb (cosmos_predict2/_src/predict2/networks/minimal_v4_dit.py:534-661): layout, fps and NTK rules."""
     import numpy as np
