@@ -1,6 +1,6 @@
 """Benchmark of the attention forward + JVP hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk|dblk|dblkf] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk|dblk|dblkf|net|netf] [--no-cpu]
 
 A "step" is one call of the hot path (re-tiling kernel + attention kernel, through the Python host and
 the C ABI) over one batch of synthetic tensors that are already resident in HBM.  Default workload: the
@@ -53,6 +53,9 @@ WORKLOADS = {
     # one whole DiT block with a tangent: adaLN modulation, self-attention, text cross-attention, MLP, gated residuals
     "dblkf": ("2B DiT block forward (inference) bf16 720p B1 T24 H44 W80 D2048 heads16 text512x1024 adaLN-LoRA256", 1, 16, 84480, 512, 128, "block_fwd", False, False),
     "dblk": ("2B DiT block fwd+JVP bf16 720p B1 T24 H44 W80 D2048 heads16 text512x1024 adaLN-LoRA256", 1, 16, 84480, 512, 128, "block", False, False),
+    # the whole 2B video-conditioned DiT (28 blocks; patch / time embedding, text projection 100352 -> 1024, final layer)
+    "netf": ("2B DiT network forward (inference) bf16 720p B1 x16x24x88x160 28 blocks D2048 heads16 text512x100352", 1, 16, 84480, 512, 128, "network_fwd", False, False),
+    "net": ("2B DiT network fwd+JVP along (x, t) bf16 720p B1 x16x24x88x160 28 blocks D2048 heads16 text512x100352", 1, 16, 84480, 512, 128, "network", False, False),
 }
 PEAK_HBM_GBS = 8000.0
 
@@ -280,6 +283,77 @@ def bench_block(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False):
     print(json.dumps(result), flush=True)
 
 
+def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False):
+    """One step = MinimalV1LVGDiT.forward_jvp (or, with ``forward_only``, its forward under no_grad) of the 2B DiT:
+    16 latent channels x 24 latent frames x 88 x 160, 2 x 2 patches -> 84480 tokens, 28 blocks."""
+    K, Kc, Kin, T, Hh, W, C, n_blocks = H * D, 1024, 100352, 24, 88, 160, 16, 28
+    assert T * (Hh // 2) * (W // 2) == L
+    torch.manual_seed(0)
+    with torch.device(dev):
+        net = pkg.MinimalV1LVGDiT(max_img_h=240, max_img_w=240, max_frames=128, in_channels=C, out_channels=C, patch_spatial=2,
+                                  patch_temporal=1, model_channels=K, num_blocks=n_blocks, num_heads=H, concat_padding_mask=True,
+                                  use_adaln_lora=True, adaln_lora_dim=256, crossattn_emb_channels=Kc,
+                                  use_crossattn_projection=True, crossattn_proj_in_channels=Kin)
+        with torch.no_grad():   # a freshly initialised network has zero modulation layers; give them something to do
+            for blk in net.blocks:
+                for mod in (blk.adaln_modulation_self_attn, blk.adaln_modulation_cross_attn, blk.adaln_modulation_mlp):
+                    mod[-1].weight.copy_(torch.randn_like(mod[-1].weight) / 64.0)
+            net.final_layer.adaln_modulation[-1].weight.copy_(torch.randn_like(net.final_layer.adaln_modulation[-1].weight) / 16.0)
+    net = net.to(dtype=torch.bfloat16).eval()
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(s, generator=g, device=dev)
+    x, tx = rn(B, C, T, Hh, W).bfloat16(), (0.1 * rn(B, C, T, Hh, W)).bfloat16()
+    ts = torch.full((B, 1), 0.6, device=dev, dtype=torch.bfloat16)
+    tts = torch.full((B, 1), 0.5, device=dev, dtype=torch.bfloat16)
+    ctx = rn(B, Mk, Kin).bfloat16()
+    cond = torch.zeros(B, 1, T, Hh, W, device=dev, dtype=torch.bfloat16)
+    cond[:, :, :1] = 1
+    pm = torch.zeros(B, 1, Hh, W, device=dev, dtype=torch.bfloat16)
+    fps = torch.full((B,), 16.0, device=dev)
+    gemm = lambda rows, k, n: 2.0 * rows * k * n
+    cin = (C + 2) * 4
+    per_block = (4 * 2 * gemm(B * L, K, K) + 6 * 2.0 * B * H * L * L * D + 2 * 2 * gemm(B * L, K, K) + 2 * gemm(B * Mk, Kc, K)
+                 + 4 * 2.0 * B * H * L * Mk * D + 2 * 2 * gemm(B * L, K, 4 * K))
+    ends = 2 * gemm(B * L, cin, K) + 2 * gemm(B * L, K, 4 * C) + gemm(B * Mk, Kin, Kc)
+    step = lambda: net.forward_jvp(x, tx, ts, tts, ctx, cond, fps=fps, padding_mask=pm)
+    if forward_only:
+        per_block = (4 * gemm(B * L, K, K) + 2 * 2.0 * B * H * L * L * D + 2 * gemm(B * L, K, K) + 2 * gemm(B * Mk, Kc, K)
+                     + 2 * 2.0 * B * H * L * Mk * D + 2 * gemm(B * L, K, 4 * K))
+        ends = gemm(B * L, cin, K) + gemm(B * L, K, 4 * C) + gemm(B * Mk, Kin, Kc)
+
+        def step():
+            with torch.no_grad():
+                return net(x, ts, ctx, cond, fps=fps, padding_mask=pm)
+    total = n_blocks * per_block + ends
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        out = step()
+    e1.record()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / args.steps
+    avg = e0.elapsed_time(e1) / args.steps
+    del out
+    achieved = total / (avg * 1e-3) / 1e12
+    result = {
+        "metric": ("DiT network forward" if forward_only else "DiT network fwd+JVP") + " TFLOP/s & % bf16 MFMA peak @ 2B 720p (L=84480, 28 blocks); ms per call",
+        "value": total / sec / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": desc_txt, "flop_per_call": total, "flop_per_block": per_block, "flop_outside_blocks": ends,
+                   "peak_memory_gb": torch.cuda.max_memory_allocated() / 1e9,
+                   "pct_of_bf16_mfma_peak": 100.0 * total / sec / 1e12 / PEAK_BF16_TFLOPS},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "whole network call (the attention kernel dominates)", "kernel_ms_avg": avg},
+    }
+    print(json.dumps(result), flush=True)
+
+
 def copy_calibration(dev):
     """One plain elementwise copy kernel that reads 1 GiB and writes 1 GiB: the known-size launch the FETCH_SIZE /
     WRITE_SIZE counters are scaled by."""
@@ -377,6 +451,8 @@ def main():
     desc_txt, B, H, Lq, Lkv, d, tangents, rms, padded = WORKLOADS[args.workload]
     if tangents == "bwd":
         return bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
+    if tangents in ("network", "network_fwd"):
+        return bench_network(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, forward_only=tangents == "network_fwd")
     if tangents in ("block", "block_fwd"):
         return bench_block(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, forward_only=tangents == "block_fwd")
     if tangents == "module":

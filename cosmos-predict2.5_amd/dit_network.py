@@ -7,7 +7,9 @@ Reference: ``MiniTrainDIT`` (cosmos_predict2/_src/predict2/networks/minimal_v4_d
 parameter names (``x_embedder.proj.1.weight``, ``t_embedder.1.linear_{1,2}``, ``t_embedding_norm.weight``,
 ``blocks.N.*``, ``final_layer.linear / adaln_modulation``, ``crossattn_proj.0``, ``img_context_proj.0``,
 ``extra_pos_embedder.pos_emb_{h,w,t}``: a reference checkpoint of the network loads as is), and
-``forward(x_B_C_T_H_W, timesteps_B_T, crossattn_emb, fps, padding_mask, img_context_emb=...)``.
+``forward(x_B_C_T_H_W, timesteps_B_T, crossattn_emb, fps, padding_mask, img_context_emb=...)``; and the
+video-conditioned subclass ``MinimalV1LVGDiT`` (networks/minimal_v1_lvg_dit.py:24-62: one more input channel for the
+condition mask, ``timestep_scale``).
 
 ``forward_jvp`` is what a consistency-distillation step needs: the network output and its derivative along a
 direction ``(tx, ttimesteps)`` in one pass (conditioning, positions and padding mask do not move).  The blocks carry the
@@ -404,3 +406,42 @@ class MiniTrainDIT(nn.Module):
             x, tx = block.forward_jvp(x, tx, emb, temb, context_input, rope, lora, tlora, extra_per_block_pos_emb=extra)
         y, ty = self.final_layer.forward_jvp(x, tx, emb, temb, lora, tlora)
         return self.unpatchify(y), self.unpatchify(ty)
+
+
+def _is_video(data_type) -> bool:
+    """The reference passes a ``DataType`` enum (VIDEO / IMAGE); its name or a plain string is accepted here."""
+    if data_type is None:
+        return True
+    return str(getattr(data_type, "name", data_type)).lower() == "video"
+
+
+class MinimalV1LVGDiT(MiniTrainDIT):
+    """Video-conditioned network (networks/minimal_v1_lvg_dit.py:24-62): the condition mask ``[B, 1, T, H, W]`` (1 on the
+    given frames) is one more input channel, zeros for image batches; timesteps are multiplied by ``timestep_scale``."""
+
+    def __init__(self, *args, timestep_scale: float = 1.0, **kwargs):
+        assert "in_channels" in kwargs, "in_channels must be provided"
+        kwargs["in_channels"] += 1
+        self.timestep_scale = timestep_scale
+        super().__init__(*args, **kwargs)
+
+    def _with_condition_mask(self, x_B_C_T_H_W, mask, data_type):
+        if _is_video(data_type):
+            return torch.cat([x_B_C_T_H_W, mask.type_as(x_B_C_T_H_W)], dim=1)
+        return torch.cat([x_B_C_T_H_W, torch.zeros_like(x_B_C_T_H_W[:, :1])], dim=1)
+
+    def forward(self, x_B_C_T_H_W, timesteps_B_T, crossattn_emb, condition_video_input_mask_B_C_T_H_W=None, fps=None,
+                padding_mask=None, data_type=None, intermediate_feature_ids=None, img_context_emb=None, **kwargs):
+        del kwargs
+        x = self._with_condition_mask(x_B_C_T_H_W, condition_video_input_mask_B_C_T_H_W, data_type)
+        return super().forward(x, timesteps_B_T * self.timestep_scale, crossattn_emb, fps=fps, padding_mask=padding_mask,
+                               intermediate_feature_ids=intermediate_feature_ids, img_context_emb=img_context_emb)
+
+    @torch.no_grad()
+    def forward_jvp(self, x_B_C_T_H_W, tx_B_C_T_H_W, timesteps_B_T, ttimesteps_B_T, crossattn_emb,
+                    condition_video_input_mask_B_C_T_H_W=None, fps=None, padding_mask=None, data_type=None, img_context_emb=None):
+        x = self._with_condition_mask(x_B_C_T_H_W, condition_video_input_mask_B_C_T_H_W, data_type)
+        tx = torch.cat([tx_B_C_T_H_W, torch.zeros_like(tx_B_C_T_H_W[:, :1])], dim=1)     # the mask does not move
+        tts = None if ttimesteps_B_T is None else ttimesteps_B_T * self.timestep_scale
+        return super().forward_jvp(x, tx, timesteps_B_T * self.timestep_scale, tts, crossattn_emb, fps=fps,
+                                   padding_mask=padding_mask, img_context_emb=img_context_emb)

@@ -141,3 +141,43 @@ def test_fresh_network_output_does_not_depend_on_time(pkg, gpu):
         b = net(x, 3 * ts, ctx, fps=fps, padding_mask=pm)
     assert torch.equal(out, a) and torch.equal(a, b)
     assert float(tout.float().abs().max()) == 0.0
+
+
+def test_video_conditioned_network(pkg, oracle, net_oracle, gpu):
+    """MinimalV1LVGDiT (minimal_v1_lvg_dit.py:24-62): the condition mask is one more input channel (zeros for an image
+    batch) and the timesteps are scaled; checked against the network oracle on the concatenated input."""
+    torch.manual_seed(23)
+    kw = dict(SMALL, use_adaln_lora=True, adaln_lora_dim=16)
+    net = pkg.MinimalV1LVGDiT(in_channels=4, timestep_scale=0.5, **kw)
+    assert net.x_embedder.proj[1].weight.shape[1] == (4 + 1 + 1) * 4
+    with torch.no_grad():
+        for blk in net.blocks:
+            for mod in (blk.adaln_modulation_self_attn, blk.adaln_modulation_cross_attn, blk.adaln_modulation_mlp):
+                mod[-1].weight.copy_(torch.randn_like(mod[-1].weight) / 4.0)
+        net.final_layer.adaln_modulation[-1].weight.copy_(torch.randn_like(net.final_layer.adaln_modulation[-1].weight) / 4.0)
+    net = net.to(device=gpu, dtype=torch.bfloat16).eval()
+    g = torch.Generator().manual_seed(24)
+    rn = lambda *s: torch.randn(*s, generator=g).bfloat16()
+    B, C, T, Hh, W = 1, 4, 2, 8, 8
+    x, tx, ctx = rn(B, C, T, Hh, W), 0.3 * rn(B, C, T, Hh, W), rn(B, 20, 96)
+    ts, tts = torch.tensor([[1.5]]).bfloat16(), torch.tensor([[0.25]]).bfloat16()
+    cond = torch.zeros(B, 1, T, Hh, W).bfloat16()
+    cond[:, :, :1] = 1
+    pm = torch.zeros(B, 1, Hh, W).bfloat16()
+    fps = torch.full((B,), 16.0)
+    d = lambda t: t.to(gpu)
+    with torch.no_grad():
+        out = net(d(x), d(ts), d(ctx), d(cond), fps=d(fps), padding_mask=d(pm))
+        out_img = net(d(x[:, :, :1]), d(ts), d(ctx), None, fps=None, padding_mask=d(pm), data_type="image")
+    out2, tout = net.forward_jvp(d(x), d(tx), d(ts), d(tts), d(ctx), d(cond), fps=d(fps), padding_mask=d(pm))
+    with torch.no_grad():
+        angles = net.pos_embedder.generate_embeddings((B, T, Hh // 2, W // 2, 0), fps=d(fps)).reshape(-1, 128).cpu()
+        angles_img = net.pos_embedder.generate_embeddings((B, 1, Hh // 2, W // 2, 0), fps=None).reshape(-1, 128).cpu()
+    run_oracle = lambda x_, tx_, a_: net_oracle.network_torch(net.state_dict(), x_, ts.float() * 0.5, ctx, num_heads=2, patch_spatial=2,
+                                                              patch_temporal=1, rope_angles=a_, padding_mask=pm, tx=tx_, ttimesteps=tts.float() * 0.5)
+    want, twant = run_oracle(torch.cat([x, cond], 1), torch.cat([tx, torch.zeros_like(cond)], 1), angles)
+    check(oracle, "out", out, want)
+    check(oracle, "out (jvp call)", out2, want)
+    check(oracle, "tout", tout, twant)
+    want_img, _ = run_oracle(torch.cat([x[:, :, :1], torch.zeros_like(cond[:, :, :1])], 1), None, angles_img)
+    check(oracle, "out (image batch)", out_img, want_img)
