@@ -177,3 +177,21 @@ def test_dweight_matches_finite_differences(nr_oracle):
     yp, _ = nr_oracle.norm_rope_closed_form(x, w + h * dirw, a)
     ym, _ = nr_oracle.norm_rope_closed_form(x, w - h * dirw, a)
     assert abs(float((dy * (yp - ym)).sum()) / (2 * h) - float((dw * dirw).sum())) < 1e-7
+
+
+def test_matches_an_independent_library_implementation(nr_oracle):
+    """The rotate-half rotary embedding and the RMSNorm of the `transformers` library (Llama: `apply_rotary_pos_emb`
+    with cos / sin tables, `LlamaRMSNorm`) on the same inputs: an implementation written by others, with the same
+    non-interleaved pairing that the reference's angle table (half vector repeated twice) is built for."""
+    llama = pytest.importorskip("transformers.models.llama.modeling_llama")
+    B, S, H, D = 2, 6, 3, 32
+    x, w = rnd((B, S, H, D), 41), 1.0 + 0.2 * rnd((D,), 42)
+    a = paired_angles(S, D, 43)
+    y, _ = nr_oracle.norm_rope_closed_form(x, w, a)
+    norm = llama.LlamaRMSNorm(D, eps=1e-6).double()
+    with torch.no_grad():
+        norm.weight.copy_(torch.from_numpy(w))
+        n = norm(torch.from_numpy(x))
+        cos, sin = torch.from_numpy(np.cos(a))[None], torch.from_numpy(np.sin(a))[None]     # [1, S, D]
+        q, _ = llama.apply_rotary_pos_emb(n, n, cos, sin, unsqueeze_dim=2)                   # [B, S, H, D] layout
+    np.testing.assert_allclose(y, q.numpy(), rtol=0, atol=2e-6)     # LlamaRMSNorm computes its statistics in fp32
