@@ -17,6 +17,8 @@ Written as one pure torch function so that ``torch.func.jvp`` gives the tangent;
 Parity status: pinned in tests/test_oracle_dit_network.py -- the patchify / unpatchify index maps by brute-force loops,
 the time embedding against explicit numpy fp64, central finite differences (fp64) for the tangent, and the
 initialisation property (final modulation zero, LoRA zero => output is ``linear(layer_norm(x))``).
+``network_grads_torch`` (torch autograd of the same function): the adjoint identity against the pinned tangent and
+finite differences in weights of every kind.
 ``t_embedding_norm`` is Transformer Engine's RMSNorm in the reference (absent here): PARITY UNPINNED against that
 library itself; it is restated as ``x * rsqrt(mean(x^2) + eps) * weight``.
 """
@@ -72,21 +74,12 @@ def unpatchify_loops(y, p: int, t: int, C: int):
     return out
 
 
-def network_torch(weights: Dict[str, "torch.Tensor"], x, timesteps, crossattn_emb, *, num_heads: int, patch_spatial: int,
-                  patch_temporal: int, rope_angles=None, padding_mask=None, img_context_emb=None, tx=None, ttimesteps=None,
-                  dtype=None):
-    """weights: the network's state dict.  x: [B, C, T, H, W]; timesteps: [B, T'] (T' = 1 or T / patch_temporal);
-    crossattn_emb: [B, Mk, Kc]; rope_angles: [T'*H'*W', head_dim]; padding_mask: [B, 1, h, w] (required iff the patch
-    embedding has one more input channel than x).  Returns (out [B, C_out, T, H, W], tout or None)."""
+def _make_network_forward(w, B, C, T, H, W, *, num_heads, p, r, a, ctx, pm, img, dt):
+    """The network as a pure function ``fwd(x [B,C,T,H,W], ts [B,T']) -> [B,C_out,T,H,W]`` of CPU torch tensors of one
+    dtype (w: state dict, possibly of tensors that require grad)."""
     import torch
     import torch.nn.functional as F
 
-    dt = dtype or torch.float32
-    f = lambda t: None if t is None else torch.as_tensor(t).detach().to("cpu", dt)
-    w = {k: f(v) for k, v in weights.items() if torch.is_floating_point(v)}
-    x, ts, ctx, a, pm, img, tx, tts = (f(t) for t in (x, timesteps, crossattn_emb, rope_angles, padding_mask, img_context_emb, tx, ttimesteps))
-    B, C, T, H, W = x.shape
-    p, r = patch_spatial, patch_temporal
     D = w["x_embedder.proj.1.weight"].shape[0]
     use_lora = "final_layer.adaln_modulation.2.weight" in w
     n_blocks = 1 + max(int(k.split(".")[1]) for k in w if k.startswith("blocks."))
@@ -133,9 +126,45 @@ def network_torch(weights: Dict[str, "torch.Tensor"], x, timesteps, crossattn_em
         y = y.reshape(B, T // r, H // p, W // p, p, p, r, C_out)
         return y.permute(0, 7, 1, 6, 2, 4, 3, 5).reshape(B, C_out, T, H, W)
 
+    return fwd
+
+
+def network_torch(weights: Dict[str, "torch.Tensor"], x, timesteps, crossattn_emb, *, num_heads: int, patch_spatial: int,
+                  patch_temporal: int, rope_angles=None, padding_mask=None, img_context_emb=None, tx=None, ttimesteps=None,
+                  dtype=None):
+    """weights: the network's state dict.  x: [B, C, T, H, W]; timesteps: [B, T'] (T' = 1 or T / patch_temporal);
+    crossattn_emb: [B, Mk, Kc]; rope_angles: [T'*H'*W', head_dim]; padding_mask: [B, 1, h, w] (required iff the patch
+    embedding has one more input channel than x).  Returns (out [B, C_out, T, H, W], tout or None)."""
+    import torch
+
+    dt = dtype or torch.float32
+    f = lambda t: None if t is None else torch.as_tensor(t).detach().to("cpu", dt)
+    w = {k: f(v) for k, v in weights.items() if torch.is_floating_point(v)}
+    x, ts, ctx, a, pm, img, tx, tts = (f(t) for t in (x, timesteps, crossattn_emb, rope_angles, padding_mask, img_context_emb, tx, ttimesteps))
+    B, C, T, H, W = x.shape
+    fwd = _make_network_forward(w, B, C, T, H, W, num_heads=num_heads, p=patch_spatial, r=patch_temporal, a=a, ctx=ctx, pm=pm, img=img, dt=dt)
     if ts.ndim == 1:
         ts = ts[:, None]
     if tx is None:
         return fwd(x, ts), None
     tts = torch.zeros_like(ts) if tts is None else tts.reshape(ts.shape)
     return torch.func.jvp(fwd, (x, ts), (tx, tts))
+
+
+def network_grads_torch(weights: Dict[str, "torch.Tensor"], x, timesteps, crossattn_emb, dout, *, num_heads: int, patch_spatial: int,
+                        patch_temporal: int, rope_angles=None, padding_mask=None, dtype=None):
+    """Reverse mode of the same function by torch autograd: (dx, {weight name: gradient}) for the cotangent ``dout`` of the
+    output.  Weights that the output does not depend on (position tables) are left out."""
+    import torch
+
+    dt = dtype or torch.float32
+    f = lambda t: None if t is None else torch.as_tensor(t).detach().to("cpu", dt)
+    w = {k: f(v).requires_grad_(True) for k, v in weights.items() if torch.is_floating_point(v) and not k.startswith("pos_embedder.")}
+    x, ts, ctx, a, pm, dout = (f(t) for t in (x, timesteps, crossattn_emb, rope_angles, padding_mask, dout))
+    x.requires_grad_(True)
+    B, C, T, H, W = x.shape
+    fwd = _make_network_forward(w, B, C, T, H, W, num_heads=num_heads, p=patch_spatial, r=patch_temporal, a=a, ctx=ctx, pm=pm, img=None, dt=dt)
+    out = fwd(x, ts if ts.ndim == 2 else ts[:, None])
+    names = list(w)
+    grads = torch.autograd.grad(out, [x] + [w[k] for k in names], grad_outputs=dout, allow_unused=True)
+    return grads[0], {k: g for k, g in zip(names, grads[1:]) if g is not None}

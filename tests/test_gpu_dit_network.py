@@ -3,7 +3,8 @@ and of its forward-mode tangent along (x, timesteps) against the CPU oracle of t
 torch.func.jvp, pinned in tests/test_oracle_dit_network.py) on the same 16-bit weights and inputs.
 
 Tolerance: the output is ``linear(layer_norm(...))`` of a stream that went through every block in 16 bits, with no
-residual carrying it: relative-L2 <= 2e-2 and max-abs <= 5e-2 * max(1, max|want|), for output and tangent alike.
+residual carrying it: relative-L2 <= 2e-2 and max-abs <= 5e-2 * max(1, max|want|), for output and tangent alike;
+weight gradients of the whole network (reverse mode through every block) relative-L2 <= 3e-2.
 """
 import math
 
@@ -181,3 +182,45 @@ def test_video_conditioned_network(pkg, oracle, net_oracle, gpu):
     check(oracle, "tout", tout, twant)
     want_img, _ = run_oracle(torch.cat([x[:, :, :1], torch.zeros_like(cond[:, :, :1])], 1), None, angles_img)
     check(oracle, "out (image batch)", out_img, want_img)
+
+
+def test_consistency_distillation_step(pkg, oracle, net_oracle, gpu):
+    """One step of the kind the forward + JVP path exists for: the tangent of the student along (dx, dt) from ``forward_jvp``
+    (no autograd: it is a stop-gradient target), then an ordinary forward and backward of
+    ``mean((F - stopgrad(F - g))^2)`` with g the normalised tangent.  The gradients of x and of every weight are checked
+    against torch autograd of the network oracle (fp32) for the same cotangent."""
+    kw = dict(SMALL, use_adaln_lora=True, adaln_lora_dim=16)
+    net = build(pkg, gpu, torch.bfloat16, 29, in_channels=4, **kw).train()
+    g = torch.Generator().manual_seed(30)
+    rn = lambda *s: torch.randn(*s, generator=g).bfloat16()
+    B, C, T, Hh, W = 1, 4, 2, 8, 8
+    x, direction, ctx = rn(B, C, T, Hh, W), rn(B, C, T, Hh, W), rn(B, 20, 96)
+    ts = torch.tensor([[0.8]]).bfloat16()
+    pm = torch.zeros(B, 1, Hh, W).bfloat16()
+    fps = torch.full((B,), 16.0)
+    d = lambda t: t.to(gpu)
+    _, tangent = net.forward_jvp(d(x), d(direction), d(ts), torch.ones_like(d(ts)), d(ctx), fps=d(fps), padding_mask=d(pm))
+    assert not tangent.requires_grad
+    gn = tangent.float() / (tangent.float().norm() + 0.1)
+    xg = d(x).requires_grad_(True)
+    out = net(xg, d(ts), d(ctx), fps=d(fps), padding_mask=d(pm))
+    loss = ((out.float() - (out.detach().float() - gn)) ** 2).mean()
+    loss.backward()
+    torch.cuda.synchronize()
+    assert math.isfinite(loss.item()) and loss.item() > 0
+    dout = (2.0 * gn / out.numel()).cpu()       # d loss / d out
+    with torch.no_grad():
+        angles = net.pos_embedder.generate_embeddings((B, T, Hh // 2, W // 2, 0), fps=d(fps)).reshape(-1, 128).cpu()
+    dx, dw = net_oracle.network_grads_torch(net.state_dict(), x, ts, ctx, dout, num_heads=2, patch_spatial=2, patch_temporal=1,
+                                            rope_angles=angles, padding_mask=pm)
+    scale = 1.0 / float(dx.abs().max())          # gradients of a mean are tiny: compare them rescaled
+    check(oracle, "dx", xg.grad.float().cpu() * scale, dx * scale, rel_l2=2e-2, max_abs=5e-2)
+    worst = ("", 0.0)
+    for name, prm in net.named_parameters():
+        assert prm.grad is not None and name in dw, name
+        want = dw[name]
+        s = 1.0 / max(float(want.abs().max()), 1e-30)
+        ma, rl = oracle.error_metrics(prm.grad.float().cpu() * s, want * s)
+        worst = max(worst, (name, rl), key=lambda z: z[1])
+        assert rl <= 3e-2, f"{name}: rel-L2 {rl}"
+    print(f"  weight gradients: worst rel-L2 {worst[1]:.3e} ({worst[0]})", flush=True)

@@ -189,3 +189,39 @@ def test_network_at_initialisation_is_projection_of_layernorm(net_oracle):
     y = (h - mu) / np.sqrt(((h - mu) ** 2).mean(-1, keepdims=True) + 1e-6) @ w["final_layer.linear.weight"].numpy().T
     np.testing.assert_allclose(out.numpy(), net_oracle.unpatchify_loops(y, p, r, C_out), atol=1e-11)
     assert tout.abs().max().item() < 1e-12
+
+
+@pytest.mark.parametrize("lora_dim", [0, 8])
+def test_network_grads_adjoint_identity_and_weight_differences(net_oracle, lora_dim):
+    """Reverse mode: <dout, J tx> = <dx, tx> with J tx from the pinned forward mode; weight gradients against central
+    differences of <dout, out> in one entry of a weight of every kind."""
+    B, C, C_out, D, H, Kc, p, r, Mk = 1, 2, 2, 16, 2, 12, 2, 1, 4
+    T, Hh, W = 2, 4, 4
+    w = make_network_weights(C=C, C_out=C_out, D=D, H=H, Kc=Kc, p=p, r=r, n_blocks=2, lora_dim=lora_dim, mask=True, extra=True, seed=21)
+    i = make_inputs(B, C, T, Hh, W, T, Mk, Kc, 22)
+    halfang = np.random.default_rng(23).standard_normal((T * 2 * 2, D // H // 2))
+    angles = np.concatenate([halfang, halfang], -1)
+    kw = dict(num_heads=H, patch_spatial=p, patch_temporal=r, rope_angles=angles, padding_mask=i["pm"], dtype=torch.float64)
+    dout = torch.randn(B, C_out, T, Hh, W, generator=torch.Generator().manual_seed(24), dtype=torch.float64)
+    dx, dw = net_oracle.network_grads_torch(w, i["x"], i["ts"], i["ctx"], dout, **kw)
+    _, tout = net_oracle.network_torch(w, i["x"], i["ts"], i["ctx"], tx=i["tx"], **kw)
+    lhs, rhs = float((dout * tout).sum()), float((dx * i["tx"]).sum())
+    assert abs(lhs - rhs) <= 1e-9 * max(1.0, abs(lhs)), (lhs, rhs)
+    assert not any(k.startswith("pos_embedder.") for k in dw)
+    eps = 1e-6
+    names = ["x_embedder.proj.1.weight", "t_embedder.1.linear_1.weight", "t_embedder.1.linear_2.weight", "t_embedding_norm.weight",
+             "blocks.0.self_attn.q_proj.weight", "blocks.1.cross_attn.k_norm.weight", "blocks.1.mlp.layer2.weight",
+             "blocks.0.adaln_modulation_mlp.1.weight", "final_layer.adaln_modulation.1.weight", "final_layer.linear.weight",
+             "extra_pos_embedder.pos_emb_h"]
+    for n, name in enumerate(names):
+        idx = tuple(int(v) % s for v, s in zip((3 + n, 5 + 2 * n), w[name].shape))
+        vals = []
+        for sign in (1, -1):
+            w2 = dict(w)
+            w2[name] = w[name].clone()
+            w2[name][idx] += sign * eps
+            out, _ = net_oracle.network_torch(w2, i["x"], i["ts"], i["ctx"], **kw)
+            vals.append(float((dout * out).sum()))
+        fd = (vals[0] - vals[1]) / (2 * eps)
+        got = float(dw[name][idx])
+        assert abs(fd - got) <= 1e-5 * max(1.0, abs(fd)), (name, idx, fd, got)
