@@ -123,3 +123,23 @@ def test_reverse_mode_through_the_module(pkg, oracle, nr_oracle, dit_oracle, gpu
         ma, rl = oracle.error_metrics(prm.grad.float().cpu(), want[name])
         print(f"  d{name}: max_abs={ma:.3e} rel_l2={rl:.3e}", flush=True)
         assert rl <= 2e-2, (name, rl)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_reference_self_attention_procedure(pkg, gpu, dtype):
+    """The reference's own live test of the module (context_parallel_test.py:64-91, backends torch / transformer_engine),
+    restated for backend "hip": same sizes, same procedure (module output against an explicit softmax(q k^T / sqrt(d)) v
+    on the q, k, v that compute_qkv returns, then output_proj), same tolerance atol = rtol = 5e-3.  The module runs in
+    16 bits here (the HIP kernels' types); the explicit path is evaluated in fp32 on those 16-bit q, k, v."""
+    torch.manual_seed(0)
+    batch_size, sequence_length, query_dim, n_heads, head_dim = 2, 16, 64, 4, 32
+    attn = pkg.Attention(query_dim=query_dim, n_heads=n_heads, head_dim=head_dim, backend="hip").to(device=gpu, dtype=dtype)
+    x_B_S_Q = torch.randn(batch_size, sequence_length, query_dim, device=gpu).to(dtype)
+    with torch.no_grad():
+        y_B_S_Q = attn(x_B_S_Q)
+        assert x_B_S_Q.shape == y_B_S_Q.shape
+        q, k, v = (t.float() for t in attn.compute_qkv(x_B_S_Q))
+        q, k, v = (t.permute(0, 2, 1, 3) for t in (head_dim ** -0.5 * q, k, v))          # B H S D
+        z = (q @ k.transpose(-2, -1)).softmax(dim=-1) @ v
+        z_B_S_Q = z.permute(0, 2, 1, 3).reshape(batch_size, sequence_length, n_heads * head_dim) @ attn.output_proj.weight.float().T
+    torch.testing.assert_close(y_B_S_Q.float(), z_B_S_Q, atol=5e-3, rtol=5e-3)
