@@ -1,6 +1,6 @@
 """Benchmark of the attention forward + JVP hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk|dblk|dblkf|net|netf] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk|dblk|dblkf|net|netf|e2e2b|e2e14b] [--no-cpu]
 
 A "step" is one call of the hot path (re-tiling kernel + attention kernel, through the Python host and
 the C ABI) over one batch of synthetic tensors that are already resident in HBM.  Default workload: the
@@ -56,6 +56,10 @@ WORKLOADS = {
     # the whole 2B video-conditioned DiT (28 blocks; patch / time embedding, text projection 100352 -> 1024, final layer)
     "netf": ("2B DiT network forward (inference) bf16 720p B1 x16x24x88x160 28 blocks D2048 heads16 text512x100352", 1, 16, 84480, 512, 128, "network_fwd", False, False),
     "net": ("2B DiT network fwd+JVP along (x, t) bf16 720p B1 x16x24x88x160 28 blocks D2048 heads16 text512x100352", 1, 16, 84480, 512, 128, "network", False, False),
+    # the reference's own end-to-end inference timing (networks/minimal_v4_dit_test_sparse_attn_e2e_speedup.py:287-375,
+    # dense self-attention cases): text-to-world MiniTrainDIT, x [1,16,24,88,160], text [1,512,1024], forward under no_grad
+    "e2e2b": ("2B text2world DiT inference forward bf16 720p B1 x16x24x88x160 28 blocks D2048 heads16 text512x1024", 1, 16, 84480, 512, 128, "e2e", False, False),
+    "e2e14b": ("14B text2world DiT inference forward bf16 720p B1 x16x24x88x160 36 blocks D5120 heads40 text512x1024", 1, 40, 84480, 512, 128, "e2e", False, False),
 }
 PEAK_HBM_GBS = 8000.0
 
@@ -283,17 +287,27 @@ def bench_block(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False):
     print(json.dumps(result), flush=True)
 
 
-def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False):
+def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False, text2world=False):
     """One step = MinimalV1LVGDiT.forward_jvp (or, with ``forward_only``, its forward under no_grad) of the 2B DiT:
-    16 latent channels x 24 latent frames x 88 x 160, 2 x 2 patches -> 84480 tokens, 28 blocks."""
-    K, Kc, Kin, T, Hh, W, C, n_blocks = H * D, 1024, 100352, 24, 88, 160, 16, 28
+    16 latent channels x 24 latent frames x 88 x 160, 2 x 2 patches -> 84480 tokens, 28 blocks.  ``text2world``: the
+    plain MiniTrainDIT of the reference's end-to-end timing script (no condition mask, text context already 1024 wide;
+    36 blocks when H = 40)."""
+    K, Kc, Kin, T, Hh, W, C, n_blocks = H * D, 1024, 100352, 24, 88, 160, 16, (36 if H == 40 else 28)
     assert T * (Hh // 2) * (W // 2) == L
     torch.manual_seed(0)
+    common = dict(max_img_h=240, max_img_w=240, max_frames=128, in_channels=C, out_channels=C, patch_spatial=2, patch_temporal=1,
+                  model_channels=K, num_blocks=n_blocks, num_heads=H, concat_padding_mask=True, use_adaln_lora=True,
+                  adaln_lora_dim=256, crossattn_emb_channels=Kc)
     with torch.device(dev):
-        net = pkg.MinimalV1LVGDiT(max_img_h=240, max_img_w=240, max_frames=128, in_channels=C, out_channels=C, patch_spatial=2,
-                                  patch_temporal=1, model_channels=K, num_blocks=n_blocks, num_heads=H, concat_padding_mask=True,
-                                  use_adaln_lora=True, adaln_lora_dim=256, crossattn_emb_channels=Kc,
-                                  use_crossattn_projection=True, crossattn_proj_in_channels=Kin)
+        torch.set_default_dtype(torch.bfloat16)     # 14B parameters: initialise them in 16 bits on the device
+        try:
+            if text2world:
+                net = pkg.MiniTrainDIT(**common)
+                Kin = Kc
+            else:
+                net = pkg.MinimalV1LVGDiT(use_crossattn_projection=True, crossattn_proj_in_channels=Kin, **common)
+        finally:
+            torch.set_default_dtype(torch.float32)
         with torch.no_grad():   # a freshly initialised network has zero modulation layers; give them something to do
             for blk in net.blocks:
                 for mod in (blk.adaln_modulation_self_attn, blk.adaln_modulation_cross_attn, blk.adaln_modulation_mlp):
@@ -311,18 +325,22 @@ def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False):
     pm = torch.zeros(B, 1, Hh, W, device=dev, dtype=torch.bfloat16)
     fps = torch.full((B,), 16.0, device=dev)
     gemm = lambda rows, k, n: 2.0 * rows * k * n
-    cin = (C + 2) * 4
+    cin = (C + (1 if text2world else 2)) * 4
     per_block = (4 * 2 * gemm(B * L, K, K) + 6 * 2.0 * B * H * L * L * D + 2 * 2 * gemm(B * L, K, K) + 2 * gemm(B * Mk, Kc, K)
                  + 4 * 2.0 * B * H * L * Mk * D + 2 * 2 * gemm(B * L, K, 4 * K))
     ends = 2 * gemm(B * L, cin, K) + 2 * gemm(B * L, K, 4 * C) + gemm(B * Mk, Kin, Kc)
     step = lambda: net.forward_jvp(x, tx, ts, tts, ctx, cond, fps=fps, padding_mask=pm)
+    if text2world:
+        assert forward_only
     if forward_only:
         per_block = (4 * gemm(B * L, K, K) + 2 * 2.0 * B * H * L * L * D + 2 * gemm(B * L, K, K) + 2 * gemm(B * Mk, Kc, K)
                      + 2 * 2.0 * B * H * L * Mk * D + 2 * gemm(B * L, K, 4 * K))
-        ends = gemm(B * L, cin, K) + gemm(B * L, K, 4 * C) + gemm(B * Mk, Kin, Kc)
+        ends = gemm(B * L, cin, K) + gemm(B * L, K, 4 * C) + (0 if text2world else gemm(B * Mk, Kin, Kc))
 
         def step():
             with torch.no_grad():
+                if text2world:
+                    return net(x, ts, ctx, fps=fps, padding_mask=pm)
                 return net(x, ts, ctx, cond, fps=fps, padding_mask=pm)
     total = n_blocks * per_block + ends
     for _ in range(args.warmup):
@@ -340,7 +358,7 @@ def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False):
     del out
     achieved = total / (avg * 1e-3) / 1e12
     result = {
-        "metric": ("DiT network forward" if forward_only else "DiT network fwd+JVP") + " TFLOP/s & % bf16 MFMA peak @ 2B 720p (L=84480, 28 blocks); ms per call",
+        "metric": ("DiT network forward" if forward_only else "DiT network fwd+JVP") + f" TFLOP/s & % bf16 MFMA peak @ 720p (L=84480, {n_blocks} blocks of {K}); ms per call",
         "value": total / sec / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
@@ -451,6 +469,8 @@ def main():
     desc_txt, B, H, Lq, Lkv, d, tangents, rms, padded = WORKLOADS[args.workload]
     if tangents == "bwd":
         return bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
+    if tangents == "e2e":
+        return bench_network(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, forward_only=True, text2world=True)
     if tangents in ("network", "network_fwd"):
         return bench_network(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, forward_only=tangents == "network_fwd")
     if tangents in ("block", "block_fwd"):
