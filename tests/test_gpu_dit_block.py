@@ -75,6 +75,12 @@ def test_block_2b_widths_reduced_length(pkg, oracle, nr_oracle, block_oracle, gp
     run(pkg, oracle, nr_oracle, block_oracle, gpu, B=1, T=3, Hh=8, W=16, D=2048, H=16, Mk=512, Kc=1024, lora_dim=256, seed=3)
 
 
+def test_block_14b_widths_reduced_length(pkg, oracle, nr_oracle, block_oracle, gpu):
+    """The 14B DiT's block (5120 wide, 40 heads of 128, adaLN-LoRA 256) on a 2 x 6 x 8 token grid: LayerNorm rows of 10
+    chunks per lane, 40 heads through the RMSNorm + RoPE kernel's head grouping."""
+    run(pkg, oracle, nr_oracle, block_oracle, gpu, B=1, T=2, Hh=6, W=8, D=5120, H=40, Mk=64, Kc=1024, lora_dim=256, seed=4)
+
+
 def test_block_with_image_context(pkg, oracle, nr_oracle, block_oracle, gpu):
     """image_context_dim: the cross-attention also attends to an image context (minimal_v4_dit.py:451-493)."""
     B, T, Hh, W, D, H, Mk, Kc, Mi, Ki = 2, 2, 4, 6, 256, 2, 20, 96, 12, 80
