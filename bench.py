@@ -305,7 +305,10 @@ def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False, 
                 net = pkg.MiniTrainDIT(**common)
                 Kin = Kc
             else:
-                net = pkg.MinimalV1LVGDiT(use_crossattn_projection=True, crossattn_proj_in_channels=Kin, **common)
+                # the released 2B rectified-flow configuration: text projection 100352 -> 1024, fp32 time embedding /
+                # modulation / final layer (configs/video2world/experiment/reason_embeddings/model_2B_reason_1p1_rectified_flow.py:321-324)
+                net = pkg.MinimalV1LVGDiT(use_crossattn_projection=True, crossattn_proj_in_channels=Kin,
+                                          use_wan_fp32_strategy=True, **common)
         finally:
             torch.set_default_dtype(torch.float32)
         with torch.no_grad():   # a freshly initialised network has zero modulation layers; give them something to do
@@ -317,8 +320,9 @@ def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False, 
     g = torch.Generator(device=dev).manual_seed(0)
     rn = lambda *s: torch.randn(s, generator=g, device=dev)
     x, tx = rn(B, C, T, Hh, W).bfloat16(), (0.1 * rn(B, C, T, Hh, W)).bfloat16()
-    ts = torch.full((B, 1), 0.6, device=dev, dtype=torch.bfloat16)
-    tts = torch.full((B, 1), 0.5, device=dev, dtype=torch.bfloat16)
+    t_dtype = torch.bfloat16 if text2world else torch.float32      # fp32 timesteps with the fp32 strategy
+    ts = torch.full((B, 1), 0.6, device=dev, dtype=t_dtype)
+    tts = torch.full((B, 1), 0.5, device=dev, dtype=t_dtype)
     ctx = rn(B, Mk, Kin).bfloat16()
     cond = torch.zeros(B, 1, T, Hh, W, device=dev, dtype=torch.bfloat16)
     cond[:, :, :1] = 1

@@ -76,17 +76,16 @@ class Block(nn.Module):
         use_wan_fp32_strategy: bool = False,
     ):
         super().__init__()
-        if use_wan_fp32_strategy:
-            raise NotImplementedError("use_wan_fp32_strategy is not built")
         self.x_dim = x_dim
+        fp32 = dict(use_wan_fp32_strategy=use_wan_fp32_strategy)
         self.layer_norm_self_attn = nn.LayerNorm(x_dim, elementwise_affine=False, eps=1e-6)
-        self.self_attn = Attention(x_dim, None, num_heads, x_dim // num_heads, qkv_format="bshd", backend=backend)
+        self.self_attn = Attention(x_dim, None, num_heads, x_dim // num_heads, qkv_format="bshd", backend=backend, **fp32)
         self.layer_norm_cross_attn = nn.LayerNorm(x_dim, elementwise_affine=False, eps=1e-6)
         if image_context_dim is None:
-            self.cross_attn = Attention(x_dim, context_dim, num_heads, x_dim // num_heads, qkv_format="bshd", backend=backend)
+            self.cross_attn = Attention(x_dim, context_dim, num_heads, x_dim // num_heads, qkv_format="bshd", backend=backend, **fp32)
         else:   # crossattn_emb is then the pair (text context, image context)
             self.cross_attn = I2VCrossAttention(x_dim, context_dim, num_heads, x_dim // num_heads,
-                                                img_latent_dim=image_context_dim, qkv_format="bshd", backend=backend)
+                                                img_latent_dim=image_context_dim, qkv_format="bshd", backend=backend, **fp32)
         self.layer_norm_mlp = nn.LayerNorm(x_dim, elementwise_affine=False, eps=1e-6)
         self.mlp = GPT2FeedForward(x_dim, int(x_dim * mlp_ratio))
 
@@ -128,10 +127,13 @@ class Block(nn.Module):
 
     # ------------------------------------------------------------------ pieces
     def _modulation(self, mod: nn.Sequential, emb_B_T_D, adaln_lora_B_T_3D, like):
-        """(shift, scale, gate), each ``[B, T, 1, 1, D]`` in the type of x (minimal_v4_dit.py:1131-1162)."""
-        m = mod(emb_B_T_D)
-        if self.use_adaln_lora:
-            m = m + adaln_lora_B_T_3D
+        """(shift, scale, gate), each ``[B, T, 1, 1, D]`` in the type of x (minimal_v4_dit.py:1131-1162).  With
+        ``use_wan_fp32_strategy`` the modulation MLP runs in fp32 (an fp32 autocast region, as in the reference) on the
+        fp32 time embedding and is rounded once, to the type of x."""
+        with self._fp32_region(emb_B_T_D):
+            m = mod(emb_B_T_D)
+            if self.use_adaln_lora:
+                m = m + adaln_lora_B_T_3D
         return tuple(c[:, :, None, None, :].type_as(like) for c in m.chunk(3, dim=-1))
 
     def _modulation_jvp(self, mod: nn.Sequential, emb, temb, lora, tlora, like):
@@ -141,9 +143,13 @@ class Block(nn.Module):
             lora = emb.new_zeros(())
         temb = torch.zeros_like(emb) if temb is None else temb
         tlora = torch.zeros_like(lora) if tlora is None else tlora
-        m, tm = torch.func.jvp(f, (emb, lora), (temb, tlora))
+        with self._fp32_region(emb):
+            m, tm = torch.func.jvp(f, (emb, lora), (temb, tlora))
         cut = lambda z: tuple(c[:, :, None, None, :].type_as(like) for c in z.chunk(3, dim=-1))
         return cut(m), cut(tm)
+
+    def _fp32_region(self, t: torch.Tensor):
+        return torch.autocast(t.device.type, enabled=self.use_wan_fp32_strategy, dtype=torch.float32)
 
     @staticmethod
     def _modulate(norm_layer, x, scale, shift):

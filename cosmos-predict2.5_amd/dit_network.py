@@ -17,8 +17,12 @@ tangent through their fused kernels (dit_block.Block.forward_jvp); the small pie
 ``[B, T, D]``) go through torch forward AD, the patch embedding and the final projection map primal and tangent
 stacked in one GEMM.
 
-Not built (refused in the constructor): sparse attention (``n_dense_blocks``, ``natten_parameters``), selective
-activation checkpointing, ``use_wan_fp32_strategy``, context parallelism.
+``use_wan_fp32_strategy`` (the released rectified-flow configurations set it): the time embedding, every modulation MLP
+and the whole final layer run in fp32 (fp32 autocast regions, as in the reference); timesteps must then arrive in fp32 and
+the output is fp32.
+
+Not built (refused in the constructor): sparse attention (``n_dense_blocks``, ``natten_parameters``); selective
+activation checkpointing is accepted and ignored; context parallelism needs a second GPU.
 """
 from __future__ import annotations
 
@@ -163,8 +167,7 @@ class FinalLayer(nn.Module):
     def __init__(self, hidden_size, spatial_patch_size, temporal_patch_size, out_channels, use_adaln_lora: bool = False,
                  adaln_lora_dim: int = 256, use_wan_fp32_strategy: bool = False):
         super().__init__()
-        if use_wan_fp32_strategy:
-            raise NotImplementedError("use_wan_fp32_strategy is not built")
+        self.use_wan_fp32_strategy = use_wan_fp32_strategy
         self.layer_norm = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
         self.linear = nn.Linear(hidden_size, spatial_patch_size * spatial_patch_size * temporal_patch_size * out_channels, bias=False)
         self.hidden_size = hidden_size
@@ -194,7 +197,18 @@ class FinalLayer(nn.Module):
             m = m + adaln_lora_B_T_3D[:, :, : 2 * self.hidden_size]     # (:969-972)
         return m
 
+    def _forward_fp32(self, x_B_T_H_W_D, emb_B_T_D, adaln_lora_B_T_3D):
+        """use_wan_fp32_strategy (:967-988): modulation, LayerNorm, modulate and the projection all in fp32 (the autocast
+        region lifts the LayerNorm input and the linear layers to fp32); fp32 output."""
+        assert emb_B_T_D.dtype == torch.float32
+        with torch.autocast(x_B_T_H_W_D.device.type, dtype=torch.float32):
+            shift, scale = self._modulation(emb_B_T_D, adaln_lora_B_T_3D).chunk(2, dim=-1)
+            n = self.layer_norm(x_B_T_H_W_D.float()) * (1 + scale[:, :, None, None, :]) + shift[:, :, None, None, :]
+            return self.linear(n)
+
     def forward(self, x_B_T_H_W_D, emb_B_T_D, adaln_lora_B_T_3D: Optional[torch.Tensor] = None):
+        if self.use_wan_fp32_strategy:
+            return self._forward_fp32(x_B_T_H_W_D, emb_B_T_D, adaln_lora_B_T_3D)
         shift, scale = self._modulation(emb_B_T_D, adaln_lora_B_T_3D).chunk(2, dim=-1)
         D = x_B_T_H_W_D.shape[-1]
         if not torch.is_grad_enabled() and x_B_T_H_W_D.is_cuda:
@@ -210,6 +224,9 @@ class FinalLayer(nn.Module):
             lora = emb.new_zeros(())
         temb = torch.zeros_like(emb) if temb is None else temb
         tlora = torch.zeros_like(lora) if tlora is None else tlora
+        if self.use_wan_fp32_strategy:     # a handful of fp32 passes over [B, T, H, W, D], once per network call
+            g = lambda x_, e, l: self._forward_fp32(x_, e, l if self.use_adaln_lora else None)
+            return torch.func.jvp(g, (x.float(), emb, lora), (tx.float(), temb, tlora))
         m, tm = torch.func.jvp(f, (emb, lora), (temb, tlora))
         D = x.shape[-1]
         (shift, scale), (tshift, tscale) = (z.type_as(x).chunk(2, dim=-1) for z in (m, tm))
@@ -264,8 +281,6 @@ class MiniTrainDIT(nn.Module):
         super().__init__()
         if n_dense_blocks != -1 or natten_parameters is not None:
             raise NotImplementedError("sparse (neighbourhood) attention is not built")
-        if use_wan_fp32_strategy:
-            raise NotImplementedError("use_wan_fp32_strategy is not built")
         if pos_emb_cls != "rope3d":
             raise ValueError(f"Unknown pos_emb_cls {pos_emb_cls}")
         del sac_config   # activation checkpointing is a training-memory policy, not part of this path
@@ -300,11 +315,12 @@ class MiniTrainDIT(nn.Module):
         self.blocks = nn.ModuleList([
             Block(x_dim=model_channels, context_dim=crossattn_emb_channels, num_heads=num_heads, mlp_ratio=mlp_ratio,
                   use_adaln_lora=use_adaln_lora, adaln_lora_dim=adaln_lora_dim, backend=atten_backend,
-                  image_context_dim=None if extra_image_context_dim is None else model_channels)
+                  image_context_dim=None if extra_image_context_dim is None else model_channels,
+                  use_wan_fp32_strategy=use_wan_fp32_strategy)
             for _ in range(num_blocks)
         ])
-        self.final_layer = FinalLayer(model_channels, patch_spatial, patch_temporal, out_channels,
-                                      use_adaln_lora=use_adaln_lora, adaln_lora_dim=adaln_lora_dim)
+        self.final_layer = FinalLayer(model_channels, patch_spatial, patch_temporal, out_channels, use_adaln_lora=use_adaln_lora,
+                                      adaln_lora_dim=adaln_lora_dim, use_wan_fp32_strategy=use_wan_fp32_strategy)
         self.t_embedding_norm = RMSNormWeight(model_channels, eps=1e-6)
         if extra_image_context_dim is not None:
             self.img_context_proj = nn.Sequential(nn.Linear(extra_image_context_dim, model_channels, bias=True), nn.GELU())
@@ -354,8 +370,11 @@ class MiniTrainDIT(nn.Module):
         return crossattn_emb
 
     def _time_embedding(self, timesteps_B_T):
-        emb, lora = self.t_embedder(timesteps_B_T)
-        return self.t_embedding_norm(emb), lora
+        """(:1610-1614) under use_wan_fp32_strategy an fp32 autocast region: with fp32 timesteps the embedding, its MLP
+        and the RMSNorm stay in fp32."""
+        with torch.autocast(timesteps_B_T.device.type, enabled=self.use_wan_fp32_strategy, dtype=torch.float32):
+            emb, lora = self.t_embedder(timesteps_B_T)
+            return self.t_embedding_norm(emb), lora
 
     # ------------------------------------------------------------------ the reference's surface
     def forward(self, x_B_C_T_H_W, timesteps_B_T, crossattn_emb, fps=None, padding_mask=None, data_type=None,

@@ -46,8 +46,9 @@ def run(pkg, oracle, net_oracle, gpu, *, B, C, T, Hh, W, Mk, Kin, dtype=torch.bf
     rn = lambda *s: torch.randn(*s, generator=g)
     x, tx = rn(B, C, T, Hh, W).to(dtype), (0.3 * rn(B, C, T, Hh, W)).to(dtype)
     Tt = T // r if per_frame_time else 1
-    ts = (torch.rand(B, Tt, generator=g) * 1.4 + 0.05).to(dtype)
-    tts = (0.2 * rn(B, Tt)).to(dtype)
+    fp32_strategy = kw.get("use_wan_fp32_strategy", False)       # timesteps then arrive in fp32 and the output is fp32
+    ts = (torch.rand(B, Tt, generator=g) * 1.4 + 0.05).to(torch.float32 if fp32_strategy else dtype)
+    tts = (0.2 * rn(B, Tt)).to(ts.dtype)
     ctx = rn(B, Mk, Kin).to(dtype)
     imgc = None if img is None else rn(B, *img).to(dtype)
     pm = (torch.rand(B, 1, Hh, W, generator=g) > 0.5).to(dtype) if kw.get("concat_padding_mask", True) else None
@@ -57,7 +58,8 @@ def run(pkg, oracle, net_oracle, gpu, *, B, C, T, Hh, W, Mk, Kin, dtype=torch.bf
         out = net(d(x), d(ts), d(ctx), fps=d(fps), padding_mask=d(pm), img_context_emb=d(imgc))
     out2, tout = net.forward_jvp(d(x), d(tx), d(ts), d(tts), d(ctx), fps=d(fps), padding_mask=d(pm), img_context_emb=d(imgc))
     torch.cuda.synchronize()
-    assert out.shape == (B, kw["out_channels"], T, Hh, W) and out.dtype == dtype and tout.shape == out.shape
+    assert out.shape == (B, kw["out_channels"], T, Hh, W) and tout.shape == out.shape
+    assert out.dtype == tout.dtype == out2.dtype == (torch.float32 if fp32_strategy else dtype)
     with torch.no_grad():
         angles = net.pos_embedder.generate_embeddings((B, T // r, Hh // p, W // p, 0), fps=d(fps)).reshape(-1, kw["model_channels"] // heads)
     want, twant = net_oracle.network_torch(net.state_dict(), x, ts, ctx, num_heads=heads, patch_spatial=p, patch_temporal=r,
@@ -76,6 +78,14 @@ SMALL = dict(max_img_h=32, max_img_w=32, max_frames=8, out_channels=4, patch_spa
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_network_small(pkg, oracle, net_oracle, gpu, lora_dim, dtype):
     run(pkg, oracle, net_oracle, gpu, B=2, C=4, T=2, Hh=8, W=12, Mk=20, Kin=96, dtype=dtype, seed=lora_dim,
+        use_adaln_lora=bool(lora_dim), adaln_lora_dim=lora_dim or 256, **SMALL)
+
+
+@pytest.mark.parametrize("lora_dim", [0, 16])
+def test_network_fp32_strategy(pkg, oracle, net_oracle, gpu, lora_dim):
+    """use_wan_fp32_strategy (set by the released rectified-flow configurations): fp32 timesteps, time embedding, modulation
+    MLPs and final layer in fp32, fp32 output (minimal_v4_dit.py:967-988, :1131, :1610)."""
+    run(pkg, oracle, net_oracle, gpu, B=2, C=4, T=2, Hh=8, W=12, Mk=20, Kin=96, seed=31 + lora_dim, use_wan_fp32_strategy=True,
         use_adaln_lora=bool(lora_dim), adaln_lora_dim=lora_dim or 256, **SMALL)
 
 

@@ -243,8 +243,7 @@ def test_dit_attention_module_mirrors_reference_surface(pkg):
         assert callable(getattr(m, name))
     with pytest.raises(AssertionError, match="Invalid backend"):
         pkg.Attention(64, backend="transformer_engine")
-    with pytest.raises(NotImplementedError):
-        pkg.Attention(64, use_wan_fp32_strategy=True)
+    assert pkg.Attention(64, use_wan_fp32_strategy=True).use_wan_fp32_strategy
     with pytest.raises(RuntimeError, match="GPU"):          # no CPU path
         with torch.no_grad():
             m.bfloat16()(torch.zeros(1, 4, 64, dtype=torch.bfloat16))
@@ -317,8 +316,8 @@ def test_dit_block_mirrors_reference_surface(pkg):
     i2v = pkg.Block(64, 48, 2, image_context_dim=32)
     assert isinstance(i2v.cross_attn, pkg.I2VCrossAttention) and i2v.cross_attn.k_img.weight.shape == (64, 32)
     assert {"cross_attn.k_img.weight", "cross_attn.v_img.weight", "cross_attn.k_img_norm.weight"} <= set(i2v.state_dict())
-    with pytest.raises(NotImplementedError):
-        pkg.Block(64, 48, 2, use_wan_fp32_strategy=True)
+    fp32 = pkg.Block(64, 48, 2, use_wan_fp32_strategy=True)
+    assert fp32.use_wan_fp32_strategy and fp32.self_attn.use_wan_fp32_strategy and fp32.cross_attn.use_wan_fp32_strategy
 
 
 def test_dit_network_mirrors_reference_surface(pkg):
@@ -347,7 +346,7 @@ def test_dit_network_mirrors_reference_surface(pkg):
     plain = pkg.MiniTrainDIT(max_img_h=16, max_img_w=16, max_frames=8, in_channels=3, out_channels=3, patch_spatial=2, patch_temporal=1,
                              model_channels=64, num_blocks=1, num_heads=2, concat_padding_mask=False)
     assert "t_embedder.1.linear_1.bias" in plain.state_dict() and "final_layer.adaln_modulation.2.weight" not in plain.state_dict()
-    for kw in (dict(n_dense_blocks=2), dict(use_wan_fp32_strategy=True), dict(natten_parameters={})):
+    for kw in (dict(n_dense_blocks=2), dict(natten_parameters={})):
         with pytest.raises(NotImplementedError):
             pkg.MiniTrainDIT(16, 16, 8, 3, 3, 2, 1, model_channels=64, num_blocks=1, num_heads=2, **kw)
 
