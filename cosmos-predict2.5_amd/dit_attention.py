@@ -75,9 +75,10 @@ class Attention(nn.Module):
         self.is_selfattn = context_dim is None
         assert backend in ["hip"], f"Invalid backend: {backend}"
         assert qkv_format == "bshd", "only the bshd format of the DiT is built"
-        # use_wan_fp32_strategy (minimal_v4_dit.py:410-412) lifts q, k to fp32 between the RMSNorm and the rotation.  The
-        # fused RMSNorm + RoPE kernel always rotates the unrounded fp32 normalised values and rounds once, when it hands q, k
-        # to the attention kernel (where the reference's attention() casts to 16 bits too): the flag changes nothing here.
+        # use_wan_fp32_strategy (minimal_v4_dit.py:410-412) lifts the 16-bit RMSNorm output of q, k to fp32 for the rotation;
+        # the attention call then casts the result to 16 bits.  The fused RMSNorm + RoPE kernel has exactly these rounding
+        # points with or without the flag (16-bit normalised value, fp32 rotation, one rounding at the store): the flag
+        # changes nothing here.
         self.backend = backend
         context_dim = query_dim if context_dim is None else context_dim
         inner_dim = head_dim * n_heads
