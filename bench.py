@@ -1,6 +1,6 @@
 """Benchmark of the attention forward + JVP hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk|dblk|dblkf|net|netf|e2e2b|e2e14b] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk|dblk|dblkf|net|netf|net14|e2e2b|e2e14b] [--no-cpu]
 
 A "step" is one call of the hot path (re-tiling kernel + attention kernel, through the Python host and
 the C ABI) over one batch of synthetic tensors that are already resident in HBM.  Default workload: the
@@ -56,6 +56,7 @@ WORKLOADS = {
     # the whole 2B video-conditioned DiT (28 blocks; patch / time embedding, text projection 100352 -> 1024, final layer)
     "netf": ("2B DiT network forward (inference) bf16 720p B1 x16x24x88x160 28 blocks D2048 heads16 text512x100352", 1, 16, 84480, 512, 128, "network_fwd", False, False),
     "net": ("2B DiT network fwd+JVP along (x, t) bf16 720p B1 x16x24x88x160 28 blocks D2048 heads16 text512x100352", 1, 16, 84480, 512, 128, "network", False, False),
+    "net14": ("14B DiT network fwd+JVP along (x, t) bf16 720p B1 x16x24x88x160 36 blocks D5120 heads40 text512x100352", 1, 40, 84480, 512, 128, "network", False, False),
     # the reference's own end-to-end inference timing (networks/minimal_v4_dit_test_sparse_attn_e2e_speedup.py:287-375,
     # dense self-attention cases): text-to-world MiniTrainDIT, x [1,16,24,88,160], text [1,512,1024], forward under no_grad
     "e2e2b": ("2B text2world DiT inference forward bf16 720p B1 x16x24x88x160 28 blocks D2048 heads16 text512x1024", 1, 16, 84480, 512, 128, "e2e", False, False),
