@@ -168,3 +168,33 @@ def test_block_reverse_mode(pkg, oracle, nr_oracle, gpu):
     check(oracle, "dx", xd.grad, want_dx)
     for name, prm in m.named_parameters():
         assert prm.grad is not None and torch.isfinite(prm.grad.float()).all(), name
+
+
+def test_block_with_image_context_reverse_mode(pkg, oracle, nr_oracle, block_oracle, gpu):
+    """Reverse mode through the image-conditioned cross-attention (two attention calls summed): the gradient of x
+    against torch autograd of the block oracle."""
+    B, T, Hh, W, D, H, Mk, Kc, Mi, Ki = 1, 2, 4, 6, 256, 2, 20, 96, 12, 80
+    torch.manual_seed(9)
+    m = pkg.Block(D, Kc, H, use_adaln_lora=True, adaln_lora_dim=16, image_context_dim=Ki)
+    m.init_weights()
+    with torch.no_grad():
+        for mod in (m.adaln_modulation_self_attn, m.adaln_modulation_cross_attn, m.adaln_modulation_mlp):
+            mod[-1].weight.copy_(torch.randn_like(mod[-1].weight) / 4.0)
+    m = m.to(device=gpu, dtype=torch.bfloat16).train()
+    g = torch.Generator().manual_seed(10)
+    r = lambda *s: torch.randn(*s, generator=g)
+    x, emb, lora = r(B, T, Hh, W, D).bfloat16(), r(B, T, D).bfloat16(), (0.3 * r(B, T, 3 * D)).bfloat16()
+    ctx, img, dout = r(B, Mk, Kc).bfloat16(), r(B, Mi, Ki).bfloat16(), r(B, T, Hh, W, D).bfloat16()
+    hd = D // H
+    angles = torch.from_numpy(nr_oracle.rope_angles_3d(T, Hh, W, hd))
+    xd = x.to(gpu).requires_grad_(True)
+    out = m(xd, emb.to(gpu), (ctx.to(gpu), img.to(gpu)), angles.reshape(-1, 1, 1, hd).to(gpu), lora.to(gpu))
+    out.backward(dout.to(gpu))
+    torch.cuda.synchronize()
+    xr = x.float().requires_grad_(True)
+    want_out, _ = block_oracle.block_torch(m.state_dict(), xr, emb, (ctx, img), angles.numpy(), H, lora, keep_graph_input=xr)
+    (want_dx,) = torch.autograd.grad(want_out, xr, grad_outputs=dout.float())
+    check(oracle, "out", out.detach(), want_out.detach())
+    check(oracle, "dx", xd.grad, want_dx)
+    for name, prm in m.named_parameters():
+        assert prm.grad is not None and torch.isfinite(prm.grad.float()).all(), name
