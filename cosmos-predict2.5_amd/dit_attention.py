@@ -73,7 +73,9 @@ class Attention(nn.Module):
     ) -> None:
         super().__init__()
         self.is_selfattn = context_dim is None
-        assert backend in ["hip"], f"Invalid backend: {backend}"
+        # "minimal_a2a" is the reference's name for the op protocol that HipAttnOp implements (a2a_cp.py:208-219): configurations
+        # written for the reference keep working.  Other libraries' kernels ("torch", "transformer_engine", ...) are not here.
+        assert backend in ["hip", "minimal_a2a"], f"Invalid backend: {backend}"
         assert qkv_format == "bshd", "only the bshd format of the DiT is built"
         # use_wan_fp32_strategy (minimal_v4_dit.py:410-412) lifts the 16-bit RMSNorm output of q, k to fp32 for the rotation;
         # the attention call then casts the result to 16 bits.  The fused RMSNorm + RoPE kernel has exactly these rounding

@@ -243,6 +243,7 @@ def test_dit_attention_module_mirrors_reference_surface(pkg):
         assert callable(getattr(m, name))
     with pytest.raises(AssertionError, match="Invalid backend"):
         pkg.Attention(64, backend="transformer_engine")
+    assert isinstance(pkg.Attention(64, backend="minimal_a2a").attn_op, pkg.HipAttnOp)    # the reference's name for this op protocol
     assert pkg.Attention(64, use_wan_fp32_strategy=True).use_wan_fp32_strategy
     with pytest.raises(RuntimeError, match="GPU"):          # no CPU path
         with torch.no_grad():
