@@ -393,6 +393,32 @@ class MiniTrainDIT(nn.Module):
         out = self.unpatchify(self.final_layer(x, emb, adaln_lora_B_T_3D=lora))
         return (out, feats) if intermediate_feature_ids else out
 
+    # ------------------------------------------------------------------ parallelism hooks of the reference (:1688-1737)
+    def enable_context_parallel(self, process_group=None):
+        """A group of one rank is accepted (nothing to exchange); more ranks need a second GPU and are refused."""
+        self.pos_embedder.enable_context_parallel(process_group=process_group)
+        ranks = None
+        if process_group is not None:
+            import torch.distributed as dist
+
+            ranks = dist.get_process_group_ranks(process_group)
+        for block in self.blocks:
+            block.set_context_parallel_group(process_group=process_group, ranks=ranks, stream=None)
+        self._is_context_parallel_enabled = True
+
+    def disable_context_parallel(self):
+        self.pos_embedder.disable_context_parallel()
+        for block in self.blocks:
+            block.set_context_parallel_group(process_group=None, ranks=None, stream=None)
+        self._is_context_parallel_enabled = False
+
+    @property
+    def is_context_parallel_enabled(self):
+        return getattr(self, "_is_context_parallel_enabled", False)
+
+    def fully_shard(self, mesh):
+        raise NotImplementedError("parameter sharding across GPUs (FSDP) is not part of this one-GPU build")
+
     # ------------------------------------------------------------------ forward mode
     @torch.no_grad()
     def forward_jvp(self, x_B_C_T_H_W, tx_B_C_T_H_W, timesteps_B_T, ttimesteps_B_T, crossattn_emb, fps=None, padding_mask=None,

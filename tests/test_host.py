@@ -351,6 +351,14 @@ def test_dit_network_mirrors_reference_surface(pkg):
         with pytest.raises(NotImplementedError):
             pkg.MiniTrainDIT(16, 16, 8, 3, 3, 2, 1, model_channels=64, num_blocks=1, num_heads=2, **kw)
 
+    assert not net.is_context_parallel_enabled
+    net.enable_context_parallel(None)
+    assert net.is_context_parallel_enabled
+    net.disable_context_parallel()
+    assert not net.is_context_parallel_enabled
+    with pytest.raises(NotImplementedError):
+        net.fully_shard(None)
+
     # host-side pieces against einops with the reference's pattern strings / explicit numpy
     x = torch.randn(2, 4, 4, 6, 8)
     pe = pkg.PatchEmbed(2, 2, in_channels=4, out_channels=16)
