@@ -1,6 +1,6 @@
 """Benchmark of the attention forward + JVP hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk|dblk|dblkf|net|netf|net14|e2e2b|e2e14b] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c3b|nr|nrb|blk|dblk|dblkf|net|netf|net14|train|e2e2b|e2e14b] [--no-cpu]
 
 A "step" is one call of the hot path (re-tiling kernel + attention kernel, through the Python host and
 the C ABI) over one batch of synthetic tensors that are already resident in HBM.  Default workload: the
@@ -56,6 +56,9 @@ WORKLOADS = {
     # the whole 2B video-conditioned DiT (28 blocks; patch / time embedding, text projection 100352 -> 1024, final layer)
     "netf": ("2B DiT network forward (inference) bf16 720p B1 x16x24x88x160 28 blocks D2048 heads16 text512x100352", 1, 16, 84480, 512, 128, "network_fwd", False, False),
     "net": ("2B DiT network fwd+JVP along (x, t) bf16 720p B1 x16x24x88x160 28 blocks D2048 heads16 text512x100352", 1, 16, 84480, 512, 128, "network", False, False),
+    # one training step of the whole 2B network: forward, backward through every block (attention backward kernels, RMSNorm +
+    # RoPE backward, library GEMMs), blocks checkpointed (sac_config) so that the activations fit
+    "train": ("2B DiT network forward + backward (block-wise activation checkpointing) bf16 720p B1 x16x24x88x160 28 blocks", 1, 16, 84480, 512, 128, "network_train", False, False),
     "net14": ("14B DiT network fwd+JVP along (x, t) bf16 720p B1 x16x24x88x160 36 blocks D5120 heads40 text512x100352", 1, 40, 84480, 512, 128, "network", False, False),
     # the reference's own end-to-end inference timing (networks/minimal_v4_dit_test_sparse_attn_e2e_speedup.py:287-375,
     # dense self-attention cases): text-to-world MiniTrainDIT, x [1,16,24,88,160], text [1,512,1024], forward under no_grad
@@ -288,7 +291,7 @@ def bench_block(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False):
     print(json.dumps(result), flush=True)
 
 
-def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False, text2world=False):
+def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False, text2world=False, train=False):
     """One step = MinimalV1LVGDiT.forward_jvp (or, with ``forward_only``, its forward under no_grad) of the 2B DiT:
     16 latent channels x 24 latent frames x 88 x 160, 2 x 2 patches -> 84480 tokens, 28 blocks.  ``text2world``: the
     plain MiniTrainDIT of the reference's end-to-end timing script (no condition mask, text context already 1024 wide;
@@ -309,7 +312,7 @@ def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False, 
                 # the released 2B rectified-flow configuration: text projection 100352 -> 1024, fp32 time embedding /
                 # modulation / final layer (configs/video2world/experiment/reason_embeddings/model_2B_reason_1p1_rectified_flow.py:321-324)
                 net = pkg.MinimalV1LVGDiT(use_crossattn_projection=True, crossattn_proj_in_channels=Kin,
-                                          use_wan_fp32_strategy=True, **common)
+                                          use_wan_fp32_strategy=True, sac_config=dict(mode="block_wise") if train else None, **common)
         finally:
             torch.set_default_dtype(torch.float32)
         with torch.no_grad():   # a freshly initialised network has zero modulation layers; give them something to do
@@ -317,7 +320,8 @@ def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False, 
                 for mod in (blk.adaln_modulation_self_attn, blk.adaln_modulation_cross_attn, blk.adaln_modulation_mlp):
                     mod[-1].weight.copy_(torch.randn_like(mod[-1].weight) / 64.0)
             net.final_layer.adaln_modulation[-1].weight.copy_(torch.randn_like(net.final_layer.adaln_modulation[-1].weight) / 16.0)
-    net = net.to(dtype=torch.bfloat16).eval()
+    net = net.to(dtype=torch.bfloat16)
+    net = net.train() if train else net.eval()
     g = torch.Generator(device=dev).manual_seed(0)
     rn = lambda *s: torch.randn(s, generator=g, device=dev)
     x, tx = rn(B, C, T, Hh, W).bfloat16(), (0.1 * rn(B, C, T, Hh, W)).bfloat16()
@@ -337,7 +341,22 @@ def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False, 
     step = lambda: net.forward_jvp(x, tx, ts, tts, ctx, cond, fps=fps, padding_mask=pm)
     if text2world:
         assert forward_only
-    if forward_only:
+    if train:
+        # model FLOP of a training step: GEMMs 3 x forward (forward, grad of input, grad of weight), attention 1 + 2.5 x forward
+        # (5 matmuls backward for 2 forward); the recomputed forward of the checkpointed blocks is not counted
+        gemm_f = 4 * gemm(B * L, K, K) + 2 * gemm(B * L, K, K) + 2 * gemm(B * Mk, Kc, K) + 2 * gemm(B * L, K, 4 * K)
+        attn_f = 2 * 2.0 * B * H * L * L * D + 2 * 2.0 * B * H * L * Mk * D
+        per_block = 3 * gemm_f + 3.5 * attn_f
+        ends = 3 * (gemm(B * L, cin, K) + gemm(B * L, K, 4 * C) + gemm(B * Mk, Kin, Kc))
+        params = [p_ for p_ in net.parameters() if p_.requires_grad]
+
+        def step():
+            for p_ in params:
+                p_.grad = None
+            out_ = net(x, ts, ctx, cond, fps=fps, padding_mask=pm)
+            out_.float().square().mean().backward()
+            return out_.detach()
+    elif forward_only:
         per_block = (4 * gemm(B * L, K, K) + 2 * 2.0 * B * H * L * L * D + 2 * gemm(B * L, K, K) + 2 * gemm(B * Mk, Kc, K)
                      + 2 * 2.0 * B * H * L * Mk * D + 2 * gemm(B * L, K, 4 * K))
         ends = gemm(B * L, cin, K) + gemm(B * L, K, 4 * C) + (0 if text2world else gemm(B * Mk, Kin, Kc))
@@ -363,7 +382,7 @@ def bench_network(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False, 
     del out
     achieved = total / (avg * 1e-3) / 1e12
     result = {
-        "metric": ("DiT network forward" if forward_only else "DiT network fwd+JVP") + f" TFLOP/s & % bf16 MFMA peak @ 720p (L=84480, {n_blocks} blocks of {K}); ms per call",
+        "metric": ("DiT network forward + backward" if train else "DiT network forward" if forward_only else "DiT network fwd+JVP") + f" TFLOP/s & % bf16 MFMA peak @ 720p (L=84480, {n_blocks} blocks of {K}); ms per call",
         "value": total / sec / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
@@ -476,6 +495,8 @@ def main():
         return bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
     if tangents == "e2e":
         return bench_network(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, forward_only=True, text2world=True)
+    if tangents == "network_train":
+        return bench_network(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, train=True)
     if tangents in ("network", "network_fwd"):
         return bench_network(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, forward_only=tangents == "network_fwd")
     if tangents in ("block", "block_fwd"):

@@ -21,8 +21,11 @@ stacked in one GEMM.
 and the whole final layer run in fp32 (fp32 autocast regions, as in the reference); timesteps must then arrive in fp32 and
 the output is fp32.
 
-Not built (refused in the constructor): sparse attention (``n_dense_blocks``, ``natten_parameters``); selective
-activation checkpointing is accepted and ignored; context parallelism needs a second GPU.
+``sac_config`` (activation checkpointing): every mode other than "none" checkpoints whole blocks (their inputs are kept,
+the block runs again in the backward pass), which is what lets a 720p training step fit.
+
+Not built (refused in the constructor): sparse attention (``n_dense_blocks``, ``natten_parameters``); context parallelism
+needs a second GPU.
 """
 from __future__ import annotations
 
@@ -31,6 +34,7 @@ from typing import Optional, Tuple
 
 import torch
 import torch.nn.functional as F
+import torch.utils.checkpoint
 from torch import nn
 
 from . import ops
@@ -238,6 +242,21 @@ class FinalLayer(nn.Module):
         return y[:b], y[b:]
 
 
+def _checkpoint_every(sac_config) -> int:
+    """Activation checkpointing of the blocks, from the reference's ``sac_config`` (a ``SACConfig``-like object or a dict
+    with ``mode`` and ``every_n_blocks``; :1660-1686).  0 = off (``None`` or mode "none"); n = every n-th block keeps only its
+    input and is run again in the backward pass.  The reference's modes choose which intermediate results of a block to
+    keep (a torch dispatcher policy); the kernels here are not dispatcher ops, so every mode means the whole block."""
+    if sac_config is None:
+        return 0
+    get = (lambda k, d: sac_config.get(k, d)) if isinstance(sac_config, dict) else (lambda k, d: getattr(sac_config, k, d))
+    mode = get("mode", "none")
+    mode = str(getattr(mode, "value", getattr(mode, "name", mode))).lower()
+    if mode in ("none", "checkpointmode.none"):
+        return 0
+    return max(1, int(get("every_n_blocks", 1)))
+
+
 class MiniTrainDIT(nn.Module):
     def __init__(
         self,
@@ -283,7 +302,7 @@ class MiniTrainDIT(nn.Module):
             raise NotImplementedError("sparse (neighbourhood) attention is not built")
         if pos_emb_cls != "rope3d":
             raise ValueError(f"Unknown pos_emb_cls {pos_emb_cls}")
-        del sac_config   # activation checkpointing is a training-memory policy, not part of this path
+        self._checkpoint_every = _checkpoint_every(sac_config)
         self.max_img_h, self.max_img_w, self.max_frames = max_img_h, max_img_w, max_frames
         self.in_channels, self.out_channels = in_channels, out_channels
         self.patch_spatial, self.patch_temporal = patch_spatial, patch_temporal
@@ -386,8 +405,14 @@ class MiniTrainDIT(nn.Module):
             timesteps_B_T = timesteps_B_T.unsqueeze(1)
         emb, lora = self._time_embedding(timesteps_B_T)
         feats = []
+        recompute = self._checkpoint_every > 0 and torch.is_grad_enabled()
         for i, block in enumerate(self.blocks):
-            x = block(x, emb, context_input, rope_emb_L_1_1_D=rope, adaln_lora_B_T_3D=lora, extra_per_block_pos_emb=extra)
+            if recompute and i % self._checkpoint_every == 0:
+                # keep only the block's input for the backward pass and run the block again there (:1660-1686)
+                x = torch.utils.checkpoint.checkpoint(block, x, emb, context_input, rope, lora, extra, use_reentrant=False,
+                                                      preserve_rng_state=False)
+            else:
+                x = block(x, emb, context_input, rope_emb_L_1_1_D=rope, adaln_lora_B_T_3D=lora, extra_per_block_pos_emb=extra)
             if intermediate_feature_ids and i in intermediate_feature_ids:
                 feats.append(x.reshape(x.shape[0], -1, x.shape[-1]))
         out = self.unpatchify(self.final_layer(x, emb, adaln_lora_B_T_3D=lora))

@@ -234,3 +234,30 @@ def test_consistency_distillation_step(pkg, oracle, net_oracle, gpu):
         worst = max(worst, (name, rl), key=lambda z: z[1])
         assert rl <= 3e-2, f"{name}: rel-L2 {rl}"
     print(f"  weight gradients: worst rel-L2 {worst[1]:.3e} ({worst[0]})", flush=True)
+
+
+def test_activation_checkpointing_gives_the_same_gradients(pkg, gpu):
+    """sac_config (minimal_v4_dit.py:1660-1686): blocks keep only their input and run again in the backward pass; the
+    recomputation is deterministic, so output and gradients are the bits of the plain run."""
+    kw = dict(SMALL, use_adaln_lora=True, adaln_lora_dim=16)
+    plain = build(pkg, gpu, torch.bfloat16, 37, in_channels=4, **kw).train()
+    ckpt = build(pkg, gpu, torch.bfloat16, 37, in_channels=4, sac_config=dict(mode="predict2_2b_720_aggressive", every_n_blocks=1), **kw).train()
+    ckpt.load_state_dict(plain.state_dict())
+    assert plain._checkpoint_every == 0 and ckpt._checkpoint_every == 1
+    g = torch.Generator().manual_seed(38)
+    rn = lambda *s: torch.randn(*s, generator=g).bfloat16().to(gpu)
+    x, ctx, dout = rn(1, 4, 2, 8, 8), rn(1, 20, 96), rn(1, 4, 2, 8, 8)
+    ts = torch.tensor([[0.7]], device=gpu, dtype=torch.bfloat16)
+    pm = torch.zeros(1, 1, 8, 8, device=gpu, dtype=torch.bfloat16)
+    fps = torch.full((1,), 16.0, device=gpu)
+    grads = []
+    for net in (plain, ckpt):
+        xg = x.clone().requires_grad_(True)
+        out = net(xg, ts, ctx, fps=fps, padding_mask=pm)
+        out.backward(dout)
+        torch.cuda.synchronize()
+        grads.append((out.detach(), xg.grad, {n: p.grad for n, p in net.named_parameters()}))
+    (o0, dx0, w0), (o1, dx1, w1) = grads
+    assert torch.equal(o0, o1) and torch.equal(dx0, dx1)
+    for name in w0:
+        assert w1[name] is not None and torch.equal(w0[name], w1[name]), name
