@@ -11,9 +11,44 @@ reads them).  The gfx950 kernels are deterministic (no atomics, fixed reduction 
 """
 from __future__ import annotations
 
+import contextlib
+import threading
+
 import torch
 
 from . import ops
+
+
+class _KeptResults(threading.local):
+    """Per host thread: where attention results (o, log-sum-exp) are being recorded, or replayed from."""
+
+    record = None     # list that every attention call appends (o, lse) to
+    replay = None     # list of (o, lse) that the next differentiable attention calls take instead of running the kernel
+
+
+_kept = _KeptResults()
+
+
+@contextlib.contextmanager
+def record_attention_results(store: list):
+    """Every ``attention()`` call inside appends its ``(o [B,H,S,D] view of [B,S,H,D] memory, lse [B,H,S])`` to ``store``."""
+    prev, _kept.record = _kept.record, store
+    try:
+        yield store
+    finally:
+        _kept.record = prev
+
+
+@contextlib.contextmanager
+def replay_attention_results(store: list):
+    """The differentiable ``attention()`` calls inside take their forward results from ``store`` (in call order) instead
+    of running the forward kernel again: activation recomputation that keeps the one expensive result of a block."""
+    prev, _kept.replay = _kept.replay, list(store)
+    try:
+        yield
+        assert not _kept.replay, "fewer attention calls in the recomputation than were recorded"
+    finally:
+        _kept.replay = prev
 
 
 class _AttentionFn(torch.autograd.Function):
@@ -22,8 +57,14 @@ class _AttentionFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, causal, softmax_scale):
-        o, _, lse = ops.fwd_jvp(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
-                                causal=causal, sm_scale=softmax_scale, out_layout="blhd", need_lse=True)
+        if _kept.replay:
+            o, lse = _kept.replay.pop(0)
+            assert o.shape == (q.shape[0], q.shape[2], q.shape[1], v.shape[3]), "recorded attention result of another call"
+        else:
+            o, _, lse = ops.fwd_jvp(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
+                                    causal=causal, sm_scale=softmax_scale, out_layout="blhd", need_lse=True)
+            if _kept.record is not None:
+                _kept.record.append((o, lse))
         ctx.save_for_backward(q, k, v, o, lse)
         ctx.causal, ctx.softmax_scale = causal, softmax_scale
         return o.transpose(1, 2)
@@ -66,8 +107,13 @@ def attention(
         return _AttentionFn.apply(q, k, v, causal, softmax_scale)   # the SDPA path of the reference is differentiable too
 
     # [B, S, H, D] -> heads-first views (no copy); the kernel writes [B, S, H, D] memory directly
-    o, _, _ = ops.fwd_jvp(
+    if _kept.replay:      # a recomputation in which q, k, v happen not to need gradients
+        return _kept.replay.pop(0)[0].transpose(1, 2)
+    recording = _kept.record is not None
+    o, _, lse = ops.fwd_jvp(
         q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
-        causal=causal, sm_scale=softmax_scale, out_layout="blhd", need_lse=False,
+        causal=causal, sm_scale=softmax_scale, out_layout="blhd", need_lse=recording,
     )
+    if recording:
+        _kept.record.append((o, lse))
     return o.transpose(1, 2)

@@ -52,6 +52,10 @@ class GPT2FeedForward(nn.Module):
             return self.layer2(ops.gelu(h, inplace=True)[0])      # inference: one fused pass, in place
         return self.layer2(self.activation(h))
 
+    def forward_plain(self, x: torch.Tensor):
+        """The tensor-library path whatever the autograd mode (what a recomputation must reproduce bit for bit)."""
+        return self.layer2(self.activation(self.layer1(x)))
+
     @torch.no_grad()
     def forward_jvp(self, x: torch.Tensor, tx: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         b = x.shape[0]
@@ -183,9 +187,14 @@ class Block(nn.Module):
         x = x_B_T_H_W_D
         if extra_per_block_pos_emb is not None:
             x = x + extra_per_block_pos_emb
-        B, T, H, W, D = x.shape
         if not torch.is_grad_enabled() and x.is_cuda:
             return self._forward_fused(x, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D, adaln_lora_B_T_3D)
+        return self._forward_unfused(x, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D, adaln_lora_B_T_3D)
+
+    def _forward_unfused(self, x, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D, adaln_lora_B_T_3D):
+        """The differentiable path: tensor-library ops around the attention kernels (x already carries the extra
+        position term)."""
+        B, T, H, W, D = x.shape
         shift, scale, gate = self._modulation(self.adaln_modulation_self_attn, emb_B_T_D, adaln_lora_B_T_3D, x)
         n = self._modulate(self.layer_norm_self_attn, x, scale, shift)
         r = self.self_attn(n.reshape(B, T * H * W, D), None, rope_emb=rope_emb_L_1_1_D).reshape(B, T, H, W, D)
@@ -196,8 +205,15 @@ class Block(nn.Module):
         x = r * gate + x
         shift, scale, gate = self._modulation(self.adaln_modulation_mlp, emb_B_T_D, adaln_lora_B_T_3D, x)
         n = self._modulate(self.layer_norm_mlp, x, scale, shift)
-        x = x + gate * self.mlp(n)
+        x = x + gate * self.mlp.forward_plain(n)
         return x
+
+    def forward_unfused(self, x_B_T_H_W_D, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D=None, adaln_lora_B_T_3D=None,
+                        extra_per_block_pos_emb=None):
+        """``forward`` through the tensor-library path whatever the autograd mode: the first pass of a recomputing
+        checkpoint runs without autograd and must produce the bits that the recomputation will."""
+        x = x_B_T_H_W_D if extra_per_block_pos_emb is None else x_B_T_H_W_D + extra_per_block_pos_emb
+        return self._forward_unfused(x, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D, adaln_lora_B_T_3D)
 
     def _forward_fused(self, x, emb, crossattn_emb, rope, lora):
         """Inference (no autograd): the same arithmetic with LayerNorm + modulation, the gated residuals and GELU each as

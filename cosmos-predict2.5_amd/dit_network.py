@@ -21,8 +21,9 @@ stacked in one GEMM.
 and the whole final layer run in fp32 (fp32 autocast regions, as in the reference); timesteps must then arrive in fp32 and
 the output is fp32.
 
-``sac_config`` (activation checkpointing): every mode other than "none" checkpoints whole blocks (their inputs are kept,
-the block runs again in the backward pass), which is what lets a 720p training step fit.
+``sac_config`` (activation checkpointing): every mode other than "none" checkpoints the blocks: a block keeps its inputs
+and the results of its attention calls, everything else is recomputed in the backward pass, which is what lets a 720p
+training step fit.
 
 Not built (refused in the constructor): sparse attention (``n_dense_blocks``, ``natten_parameters``); context parallelism
 needs a second GPU.
@@ -34,10 +35,10 @@ from typing import Optional, Tuple
 
 import torch
 import torch.nn.functional as F
-import torch.utils.checkpoint
 from torch import nn
 
 from . import ops
+from .attention import record_attention_results, replay_attention_results
 from .dit_block import Block
 from .rope_position import VideoRopePosition3DEmb
 
@@ -242,11 +243,41 @@ class FinalLayer(nn.Module):
         return y[:b], y[b:]
 
 
+class _BlockRecompute(torch.autograd.Function):
+    """Activation checkpoint of one block that keeps the attention results: the forward pass runs the block without
+    autograd and keeps its inputs plus (o, log-sum-exp) of its attention calls (0.7 GB per block at the 2B 720p shape, where
+    the forward attention kernels are 85 % of the block); the backward pass runs the block again with autograd,
+    taking those results instead of launching the forward kernels, and back-propagates through it.  The reference's
+    selective modes make the same choice with a dispatcher policy (:181-198, :1660-1686).  Restriction of this kind of
+    checkpoint: use ``loss.backward()`` (``torch.autograd.grad`` with respect to parameters inside does not see them)."""
+
+    @staticmethod
+    def forward(ctx, block, x, emb, ctx_text, ctx_img, rope, lora, extra):
+        kept = []
+        context = ctx_text if ctx_img is None else (ctx_text, ctx_img)
+        with torch.no_grad(), record_attention_results(kept):
+            out = block.forward_unfused(x, emb, context, rope, lora, extra)
+        ctx.block, ctx.kept = block, kept
+        ctx.inputs = (x, emb, ctx_text, ctx_img, rope, lora, extra)
+        return out
+
+    @staticmethod
+    def backward(ctx, gout):
+        ins = [None if t is None else t.detach().requires_grad_(t.requires_grad) for t in ctx.inputs]
+        x, emb, ctx_text, ctx_img, rope, lora, extra = ins
+        context = ctx_text if ctx_img is None else (ctx_text, ctx_img)
+        with torch.enable_grad(), replay_attention_results(ctx.kept):
+            out = ctx.block.forward_unfused(x, emb, context, rope, lora, extra)
+        ctx.kept = None
+        torch.autograd.backward(out, gout)
+        return (None,) + tuple(None if t is None else t.grad for t in ins)
+
+
 def _checkpoint_every(sac_config) -> int:
     """Activation checkpointing of the blocks, from the reference's ``sac_config`` (a ``SACConfig``-like object or a dict
-    with ``mode`` and ``every_n_blocks``; :1660-1686).  0 = off (``None`` or mode "none"); n = every n-th block keeps only its
-    input and is run again in the backward pass.  The reference's modes choose which intermediate results of a block to
-    keep (a torch dispatcher policy); the kernels here are not dispatcher ops, so every mode means the whole block."""
+    with ``mode`` and ``every_n_blocks``; :1660-1686).  0 = off (``None`` or mode "none"); n = every n-th block is
+    checkpointed (``_BlockRecompute``).  The reference's modes choose which intermediate results of a block to keep (a
+    torch dispatcher policy); here every mode keeps the same ones: the block's inputs and its attention results."""
     if sac_config is None:
         return 0
     get = (lambda k, d: sac_config.get(k, d)) if isinstance(sac_config, dict) else (lambda k, d: getattr(sac_config, k, d))
@@ -407,10 +438,11 @@ class MiniTrainDIT(nn.Module):
         feats = []
         recompute = self._checkpoint_every > 0 and torch.is_grad_enabled()
         for i, block in enumerate(self.blocks):
-            if recompute and i % self._checkpoint_every == 0:
-                # keep only the block's input for the backward pass and run the block again there (:1660-1686)
-                x = torch.utils.checkpoint.checkpoint(block, x, emb, context_input, rope, lora, extra, use_reentrant=False,
-                                                      preserve_rng_state=False)
+            text, img = context_input if isinstance(context_input, tuple) else (context_input, None)
+            # (a checkpoint whose inputs carry no gradient would never be asked to run its backward pass)
+            if recompute and i % self._checkpoint_every == 0 and any(
+                    t is not None and t.requires_grad for t in (x, emb, text, img, lora, extra)):
+                x = _BlockRecompute.apply(block, x, emb, text, img, rope, lora, extra)
             else:
                 x = block(x, emb, context_input, rope_emb_L_1_1_D=rope, adaln_lora_B_T_3D=lora, extra_per_block_pos_emb=extra)
             if intermediate_feature_ids and i in intermediate_feature_ids:

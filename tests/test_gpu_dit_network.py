@@ -237,8 +237,9 @@ def test_consistency_distillation_step(pkg, oracle, net_oracle, gpu):
 
 
 def test_activation_checkpointing_gives_the_same_gradients(pkg, gpu):
-    """sac_config (minimal_v4_dit.py:1660-1686): blocks keep only their input and run again in the backward pass; the
-    recomputation is deterministic, so output and gradients are the bits of the plain run."""
+    """sac_config (minimal_v4_dit.py:1660-1686): blocks keep their inputs and their attention results and run again in the
+    backward pass (without launching the forward attention kernels again); the recomputation is deterministic, so the
+    output, the gradient of x and the gradients of the blocks' weights are the bits of the plain run."""
     kw = dict(SMALL, use_adaln_lora=True, adaln_lora_dim=16)
     plain = build(pkg, gpu, torch.bfloat16, 37, in_channels=4, **kw).train()
     ckpt = build(pkg, gpu, torch.bfloat16, 37, in_channels=4, sac_config=dict(mode="predict2_2b_720_aggressive", every_n_blocks=1), **kw).train()
@@ -260,4 +261,11 @@ def test_activation_checkpointing_gives_the_same_gradients(pkg, gpu):
     (o0, dx0, w0), (o1, dx1, w1) = grads
     assert torch.equal(o0, o1) and torch.equal(dx0, dx1)
     for name in w0:
-        assert w1[name] is not None and torch.equal(w0[name], w1[name]), name
+        assert w1[name] is not None, name
+        if name.startswith(("t_embedder.", "t_embedding_norm.")):
+            # the time embedding feeds every block: its gradient is a sum over the blocks, which the two runs add up in 16
+            # bits in different orders
+            a, b = w0[name].float(), w1[name].float()
+            assert float((a - b).norm() / a.norm()) <= 1e-2, name
+        else:
+            assert torch.equal(w0[name], w1[name]), name
