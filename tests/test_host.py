@@ -461,3 +461,38 @@ def test_bench_refuses_more_than_one_gpu():
 
     r = subprocess.run([sys.executable, os.path.join(entry.REPO_ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_checkpoint_configuration_and_kept_attention_results_bookkeeping(pkg):
+    """sac_config parsing (object, dict, enum-valued mode) and the record / replay contexts of attention results: state is
+    per thread, restored on exit, and a recomputation that makes fewer attention calls than were recorded is an error."""
+    import enum
+    import threading
+    from types import SimpleNamespace
+
+    class Mode(enum.Enum):
+        NONE = "none"
+        BLOCK_WISE = "block_wise"
+
+    every = pkg.dit_network._checkpoint_every
+    assert every(None) == 0 and every(dict(mode="none")) == 0 and every(SimpleNamespace(mode=Mode.NONE, every_n_blocks=3)) == 0
+    assert every(dict(mode="predict2_2b_720_aggressive")) == 1 and every(SimpleNamespace(mode=Mode.BLOCK_WISE, every_n_blocks=2)) == 2
+    att = pkg.attention
+    store = []
+    with att.record_attention_results(store):
+        assert att._kept.record is store
+        seen = []
+        t = threading.Thread(target=lambda: seen.append(att._kept.record))
+        t.start(); t.join()
+        assert seen == [None]                      # another thread does not record into this one's list
+        with att.record_attention_results([]) as inner:
+            assert att._kept.record is inner
+        assert att._kept.record is store
+    assert att._kept.record is None
+    with att.replay_attention_results([]):
+        assert att._kept.replay == []
+    assert att._kept.replay is None
+    with pytest.raises(AssertionError, match="fewer attention calls"):
+        with att.replay_attention_results([("o", "lse")]):
+            pass
+    assert att._kept.replay is None
