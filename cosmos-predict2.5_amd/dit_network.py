@@ -268,7 +268,6 @@ class _BlockRecompute(torch.autograd.Function):
         context = ctx_text if ctx_img is None else (ctx_text, ctx_img)
         with torch.enable_grad(), replay_attention_results(ctx.kept):
             out = ctx.block.forward_unfused(x, emb, context, rope, lora, extra)
-        ctx.kept = None
         torch.autograd.backward(out, gout)
         return (None,) + tuple(None if t is None else t.grad for t in ins)
 
