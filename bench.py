@@ -35,7 +35,10 @@ PEAK_BF16_TFLOPS = 256 * 4096 * 2.4e9 / 1e12
 # file (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB; factors calibrated with the 1 GiB copy of --copy-calib).
 # Summaries: profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt.  None = not profiled.
 # nr: norm_rope_kernel, profiles/norm_rope_kernel_bf16_d128_workload_nr.txt.
-MEASURED_TRAFFIC_BYTES = {"c3": (2 * 3.889e7 + 710400) * 1024, "nr": (2 * 359158.94 + 675840.03) * 1024}
+# c2: attn_fwd_sym_kernel, profiles/attn_fwd_sym_kernel_bf16_d128_workload_c2.txt.  c3b: the two attn_bwd_kernel launches together,
+# profiles/attn_bwd_kernel_bf16_d128_workload_c3b.txt.
+MEASURED_TRAFFIC_BYTES = {"c3": (2 * 3.889e7 + 710400) * 1024, "nr": (2 * 359158.94 + 675840.03) * 1024,
+                          "c2": (2 * 1.733e6 + 1.997e5) * 1024, "c3b": (2 * (1.467e7 + 4.082e7) + 3.523e5 + 7.045e5) * 1024}
 
 WORKLOADS = {
     # name: (description, B, H, Lq, Lkv, d, tangents, rms-normed q/k, key-padding)
@@ -173,7 +176,7 @@ def bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d):
         "config": {"workload": desc_txt, "B": B, "H": H, "Lq": Lq, "Lkv": Lkv, "d": d, "flop_per_call": flops,
                    "executed_matmuls": 7, "pct_of_bf16_mfma_peak": 100.0 * flops / sec / 1e12 / PEAK_BF16_TFLOPS},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get("c3b"),
                      "kernel": "cosmos_attn_bwd (attn_bwd_kernel dK/dV + dQ, 3 small launches)", "kernel_ms_avg": avg, "kernel_ms_min": min(ms)},
     }
     print(json.dumps(result), flush=True)
