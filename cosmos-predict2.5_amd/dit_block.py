@@ -20,10 +20,64 @@ import math
 from typing import Optional, Tuple
 
 import torch
+import torch.nn.functional as F
 from torch import nn
 
 from . import ops
 from .dit_attention import Attention, I2VCrossAttention
+
+
+class _LnModulateFn(torch.autograd.Function):
+    """``LayerNorm(x) * (1 + scale) + shift`` as the fused pass, differentiable: the backward pass recomputes the
+    expression in fp32 with tensor-library ops and takes their gradients (x ``[B, T, H, W, D]``, shift / scale
+    ``[B, T, 1, 1, D]``)."""
+
+    @staticmethod
+    def forward(ctx, x, shift, scale, eps):
+        D = x.shape[-1]
+        y, _ = ops.ln_modulate(x, shift.reshape(-1, D), scale.reshape(-1, D), eps=eps)
+        ctx.save_for_backward(x, shift, scale)
+        ctx.eps = eps
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, shift, scale = ctx.saved_tensors
+        with torch.enable_grad():
+            xf, sh, sc = (t.detach().float().requires_grad_(True) for t in (x, shift, scale))
+            y = F.layer_norm(xf, (x.shape[-1],), eps=ctx.eps) * (1 + sc) + sh
+        dx, dsh, dsc = torch.autograd.grad(y, (xf, sh, sc), dy.float())
+        return dx.to(x.dtype), dsh.to(shift.dtype), dsc.to(scale.dtype), None
+
+
+class _GatedResidualFn(torch.autograd.Function):
+    """``x + gate * res`` as the fused pass, differentiable (gate ``[B, T, 1, 1, D]``)."""
+
+    @staticmethod
+    def forward(ctx, x, res, gate):
+        out, _ = ops.gated_residual(x, res, gate.reshape(-1, x.shape[-1]))
+        ctx.save_for_backward(res, gate)
+        return out
+
+    @staticmethod
+    def backward(ctx, dy):
+        res, gate = ctx.saved_tensors
+        dgate = (dy.float() * res.float()).sum(dim=(2, 3), keepdim=True).to(gate.dtype)
+        return dy, dy * gate, dgate
+
+
+class _GeluFn(torch.autograd.Function):
+    """Exact GELU as the fused pass, differentiable."""
+
+    @staticmethod
+    def forward(ctx, h):
+        ctx.save_for_backward(h)
+        return ops.gelu(h)[0]
+
+    @staticmethod
+    def backward(ctx, dy):
+        (h,) = ctx.saved_tensors
+        return torch.ops.aten.gelu_backward(dy, h, approximate="none")
 
 
 class GPT2FeedForward(nn.Module):
@@ -48,13 +102,11 @@ class GPT2FeedForward(nn.Module):
 
     def forward(self, x: torch.Tensor):
         h = self.layer1(x)
-        if not torch.is_grad_enabled() and h.is_cuda and h.numel() % 8 == 0:
+        if h.is_cuda and h.numel() % 8 == 0 and h.dtype in (torch.bfloat16, torch.float16):
+            if torch.is_grad_enabled() and h.requires_grad:
+                return self.layer2(_GeluFn.apply(h))
             return self.layer2(ops.gelu(h, inplace=True)[0])      # inference: one fused pass, in place
         return self.layer2(self.activation(h))
-
-    def forward_plain(self, x: torch.Tensor):
-        """The tensor-library path whatever the autograd mode (what a recomputation must reproduce bit for bit)."""
-        return self.layer2(self.activation(self.layer1(x)))
 
     @torch.no_grad()
     def forward_jvp(self, x: torch.Tensor, tx: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -156,10 +208,6 @@ class Block(nn.Module):
         return torch.autocast(t.device.type, enabled=self.use_wan_fp32_strategy, dtype=torch.float32)
 
     @staticmethod
-    def _modulate(norm_layer, x, scale, shift):
-        return norm_layer(x) * (1 + scale) + shift
-
-    @staticmethod
     def _modulate_jvp(norm_layer, x, tx, mod, tmod):
         """LayerNorm + modulation of x and its tangent (one fused pass), written into the two halves of one buffer so
         that the projections that follow map both in one GEMM without a copy."""
@@ -189,31 +237,24 @@ class Block(nn.Module):
             x = x + extra_per_block_pos_emb
         if not torch.is_grad_enabled() and x.is_cuda:
             return self._forward_fused(x, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D, adaln_lora_B_T_3D)
-        return self._forward_unfused(x, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D, adaln_lora_B_T_3D)
+        return self._forward_autograd(x, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D, adaln_lora_B_T_3D)
 
-    def _forward_unfused(self, x, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D, adaln_lora_B_T_3D):
-        """The differentiable path: tensor-library ops around the attention kernels (x already carries the extra
-        position term)."""
+    def _forward_autograd(self, x, emb, crossattn_emb, rope, lora):
+        """The differentiable path: the same kernels as the inference path (so both give the same bits), each behind an
+        autograd rule -- attention and RMSNorm + RoPE through their HIP backward kernels, the elementwise passes through
+        fp32 tensor-library arithmetic."""
         B, T, H, W, D = x.shape
-        shift, scale, gate = self._modulation(self.adaln_modulation_self_attn, emb_B_T_D, adaln_lora_B_T_3D, x)
-        n = self._modulate(self.layer_norm_self_attn, x, scale, shift)
-        r = self.self_attn(n.reshape(B, T * H * W, D), None, rope_emb=rope_emb_L_1_1_D).reshape(B, T, H, W, D)
-        x = x + gate * r
-        shift, scale, gate = self._modulation(self.adaln_modulation_cross_attn, emb_B_T_D, adaln_lora_B_T_3D, x)
-        n = self._modulate(self.layer_norm_cross_attn, x, scale, shift)
-        r = self.cross_attn(n.reshape(B, T * H * W, D), crossattn_emb, rope_emb=rope_emb_L_1_1_D).reshape(B, T, H, W, D)
-        x = r * gate + x
-        shift, scale, gate = self._modulation(self.adaln_modulation_mlp, emb_B_T_D, adaln_lora_B_T_3D, x)
-        n = self._modulate(self.layer_norm_mlp, x, scale, shift)
-        x = x + gate * self.mlp.forward_plain(n)
+        for name, norm, sub in (("self_attn", self.layer_norm_self_attn, self.self_attn),
+                                ("cross_attn", self.layer_norm_cross_attn, self.cross_attn),
+                                ("mlp", self.layer_norm_mlp, self.mlp)):
+            shift, scale, gate = self._modulation(getattr(self, "adaln_modulation_" + name), emb, lora, x)
+            n = _LnModulateFn.apply(x, shift, scale, norm.eps)
+            if name == "mlp":
+                r = sub(n)
+            else:
+                r = sub(n.reshape(B, T * H * W, D), None if name == "self_attn" else crossattn_emb, rope_emb=rope)
+            x = _GatedResidualFn.apply(x, r.reshape(x.shape), gate)
         return x
-
-    def forward_unfused(self, x_B_T_H_W_D, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D=None, adaln_lora_B_T_3D=None,
-                        extra_per_block_pos_emb=None):
-        """``forward`` through the tensor-library path whatever the autograd mode: the first pass of a recomputing
-        checkpoint runs without autograd and must produce the bits that the recomputation will."""
-        x = x_B_T_H_W_D if extra_per_block_pos_emb is None else x_B_T_H_W_D + extra_per_block_pos_emb
-        return self._forward_unfused(x, emb_B_T_D, crossattn_emb, rope_emb_L_1_1_D, adaln_lora_B_T_3D)
 
     def _forward_fused(self, x, emb, crossattn_emb, rope, lora):
         """Inference (no autograd): the same arithmetic with LayerNorm + modulation, the gated residuals and GELU each as

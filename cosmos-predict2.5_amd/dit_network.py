@@ -256,7 +256,7 @@ class _BlockRecompute(torch.autograd.Function):
         kept = []
         context = ctx_text if ctx_img is None else (ctx_text, ctx_img)
         with torch.no_grad(), record_attention_results(kept):
-            out = block.forward_unfused(x, emb, context, rope, lora, extra)
+            out = block(x, emb, context, rope, lora, extra)
         ctx.block, ctx.kept = block, kept
         ctx.inputs = (x, emb, ctx_text, ctx_img, rope, lora, extra)
         return out
@@ -267,7 +267,7 @@ class _BlockRecompute(torch.autograd.Function):
         x, emb, ctx_text, ctx_img, rope, lora, extra = ins
         context = ctx_text if ctx_img is None else (ctx_text, ctx_img)
         with torch.enable_grad(), replay_attention_results(ctx.kept):
-            out = ctx.block.forward_unfused(x, emb, context, rope, lora, extra)
+            out = ctx.block(x, emb, context, rope, lora, extra)
         torch.autograd.backward(out, gout)
         return (None,) + tuple(None if t is None else t.grad for t in ins)
 
