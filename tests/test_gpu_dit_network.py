@@ -269,3 +269,33 @@ def test_activation_checkpointing_gives_the_same_gradients(pkg, gpu):
             assert float((a - b).norm() / a.norm()) <= 1e-2, name
         else:
             assert torch.equal(w0[name], w1[name]), name
+
+
+def test_activation_checkpointing_with_every_option(pkg, gpu):
+    """The block checkpoint with a learned position term, a projected text context and an image context (all of them carry
+    gradients into the checkpointed blocks), every second block checkpointed: gradients of all weights as in the plain run."""
+    kw = dict(SMALL, patch_temporal=2, extra_per_block_abs_pos_emb=True, use_crossattn_projection=True, crossattn_proj_in_channels=80,
+              extra_image_context_dim=48, concat_padding_mask=False, use_adaln_lora=True, adaln_lora_dim=16, num_blocks=3)
+    plain = build(pkg, gpu, torch.bfloat16, 41, in_channels=3, **kw).train()
+    ckpt = build(pkg, gpu, torch.bfloat16, 41, in_channels=3, sac_config=dict(mode="block_wise", every_n_blocks=2), **kw).train()
+    ckpt.load_state_dict(plain.state_dict())
+    g = torch.Generator().manual_seed(42)
+    rn = lambda *s: torch.randn(*s, generator=g).bfloat16().to(gpu)
+    x, ctx, img, dout = rn(1, 3, 4, 8, 8), rn(1, 20, 80), rn(1, 12, 48), rn(1, 4, 4, 8, 8)
+    ts = torch.tensor([[0.7, 0.9]], device=gpu, dtype=torch.bfloat16)
+    fps = torch.full((1,), 16.0, device=gpu)
+    grads = []
+    for net in (plain, ckpt):
+        out = net(x, ts, ctx, fps=fps, img_context_emb=img)
+        out.backward(dout)
+        torch.cuda.synchronize()
+        grads.append((out.detach(), {n: p.grad for n, p in net.named_parameters()}))
+    (o0, w0), (o1, w1) = grads
+    assert torch.equal(o0, o1)
+    for name in w0:
+        assert w0[name] is not None and w1[name] is not None, name
+        a, b = w0[name].float(), w1[name].float()
+        if name.startswith("blocks."):
+            assert torch.equal(a, b), name
+        else:       # sums over the blocks, added up in 16 bits in another order
+            assert float((a - b).norm() / a.norm().clamp_min(1e-30)) <= 1e-2, name
