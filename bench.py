@@ -31,14 +31,17 @@ import __graft_entry__ as entry  # noqa: E402
 # MI355X dense bf16 MFMA peak: 256 CU x 4096 FLOP/clk/CU x 2.4 GHz
 PEAK_BF16_TFLOPS = 256 * 4096 * 2.4e9 / 1e12
 
-# HBM-side bytes per launch of attn_fwd_jvp_kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# file (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB; factors calibrated with the 1 GiB copy of --copy-calib).
-# Summaries: profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt.  None = not profiled.
-# nr: norm_rope_kernel, profiles/norm_rope_kernel_bf16_d128_workload_nr.txt.
-# c2: attn_fwd_sym_kernel, profiles/attn_fwd_sym_kernel_bf16_d128_workload_c2.txt.  c3b: the two attn_bwd_kernel launches together,
-# profiles/attn_bwd_kernel_bf16_d128_workload_c3b.txt.
-MEASURED_TRAFFIC_BYTES = {"c3": (2 * 3.889e7 + 710400) * 1024, "nr": (2 * 359158.94 + 675840.03) * 1024,
-                          "c2": (2 * 1.733e6 + 1.997e5) * 1024, "c3b": (2 * (1.467e7 + 4.082e7) + 3.523e5 + 7.045e5) * 1024}
+# HBM-side bytes per launch of the dominant kernel.  NOT measured by this program: each figure is copied from a
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE session of this file (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB; factors calibrated
+# with the 1 GiB copy of --copy-calib) whose summary is the named file; the JSON line carries the file name next to the
+# number ("traffic_source").  A workload without a counter run reports null.
+MEASURED_TRAFFIC_BYTES = {
+    "c3": ((2 * 3.889e7 + 710400) * 1024, "profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt"),
+    "nr": ((2 * 359158.94 + 675840.03) * 1024, "profiles/norm_rope_kernel_bf16_d128_workload_nr.txt"),
+    "c2": ((2 * 1.733e6 + 1.997e5) * 1024, "profiles/attn_fwd_sym_kernel_bf16_d128_workload_c2.txt"),
+    "c3b": ((2 * (1.467e7 + 4.082e7) + 3.523e5 + 7.045e5) * 1024, "profiles/attn_bwd_kernel_bf16_d128_workload_c3b.txt"),
+}
+_NO_TRAFFIC = (None, None)
 
 WORKLOADS = {
     # name: (description, B, H, Lq, Lkv, d, tangents, rms-normed q/k, key-padding)
@@ -123,6 +126,12 @@ def cpu_baseline(oracle, H, Lkv, d, tangents, rows=512, seed=0):
     }
 
 
+def rope_angles(pkg, dev, T, Hh, W, D):
+    """The rotary angle table [T*Hh*W, D] fp32 of the DiT's positional embedder (the package's own host-side class)."""
+    pe = pkg.VideoRopePosition3DEmb(head_dim=D, len_h=Hh, len_w=W, len_t=T, enable_fps_modulation=False).to(dev)
+    return pe.generate_embeddings((1, T, Hh, W, D)).reshape(T * Hh * W, D).contiguous()
+
+
 def gemm_reference(dev):
     """TFLOP/s of torch.matmul (hipBLASLt) on square bf16 operands: context for the roofline fraction."""
     out = {}
@@ -143,24 +152,24 @@ def gemm_reference(dev):
     return out
 
 
-def bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d):
+def bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, steps, warmup):
     """One step = cosmos_attn_bwd (statistics, two stream re-tilings, dK/dV kernel, dQ kernel) through the Python host."""
     q, k, v, dout, _, _ = make_device_inputs(B, H, Lq, Lkv, d, "q", False, dev)
     dout = dout * 10.0   # ~N(0, 1)
     o, _, lse = pkg.fwd_jvp(q, k, v)
     flops = 5 * 2.0 * B * H * Lq * Lkv * d   # the reference's accounting: 5 matmuls
     step = lambda: pkg.bwd(q, k, v, o, lse, dout)
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         out = step()
     torch.cuda.synchronize()
-    sec = (time.perf_counter() - t0) / args.steps
+    sec = (time.perf_counter() - t0) / steps
     del out
     ms = []
-    for i in range(args.steps):
+    for i in range(steps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(); out = step(); e1.record()
         torch.cuda.synchronize()
@@ -170,21 +179,20 @@ def bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d):
     achieved = flops / (avg * 1e-3) / 1e12
     result = {
         "metric": "attn backward TFLOP/s & % bf16 MFMA peak @ 2B 720p (L=84480); ms per call",
-        "value": flops / sec / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": flops / sec / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": desc_txt, "B": B, "H": H, "Lq": Lq, "Lkv": Lkv, "d": d, "flop_per_call": flops,
                    "executed_matmuls": 7, "pct_of_bf16_mfma_peak": 100.0 * flops / sec / 1e12 / PEAK_BF16_TFLOPS},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get("c3b"),
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["c3b"][0], "traffic_source": MEASURED_TRAFFIC_BYTES["c3b"][1],
                      "kernel": "cosmos_attn_bwd (attn_bwd_kernel dK/dV + dQ, 3 small launches)", "kernel_ms_avg": avg, "kernel_ms_min": min(ms)},
     }
-    print(json.dumps(result), flush=True)
+    return result
 
 
 def bench_module(args, pkg, dev, desc_txt, B, H, L, D):
     """One step = Attention.forward_jvp(x, tx, rope_emb) of the 2B DiT's self-attention module (K = H * D)."""
-    nro = entry.load_norm_rope_oracle()
     K = H * D
     torch.manual_seed(0)
     m = pkg.Attention(K, None, n_heads=H, head_dim=D)
@@ -193,7 +201,7 @@ def bench_module(args, pkg, dev, desc_txt, B, H, L, D):
     g = torch.Generator(device=dev).manual_seed(0)
     x = torch.randn((B, L, K), generator=g, device=dev).to(torch.bfloat16)
     tx = (torch.randn((B, L, K), generator=g, device=dev) * 0.1).to(torch.bfloat16)
-    rope = torch.from_numpy(nro.rope_angles_3d(24, 44, 80, D)).to(dev).reshape(L, 1, 1, D)
+    rope = rope_angles(pkg, dev, 24, 44, 80, D).reshape(L, 1, 1, D)
     flops_gemm = 4 * 2 * 2.0 * B * L * K * K              # q, k, v, output projections on primal and tangent
     flops_attn = 6 * 2.0 * B * H * L * L * D
     flops = flops_gemm + flops_attn
@@ -230,7 +238,6 @@ def bench_module(args, pkg, dev, desc_txt, B, H, L, D):
 def bench_block(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False):
     """One step = Block.forward_jvp (or, with ``forward_only``, Block.forward under no_grad) of the 2B DiT's transformer
     block at the 720p token grid."""
-    nro = entry.load_norm_rope_oracle()
     K, Kc, T, Hh, W = H * D, 1024, 24, 44, 80
     assert T * Hh * W == L
     torch.manual_seed(0)
@@ -246,7 +253,7 @@ def bench_block(args, pkg, dev, desc_txt, B, H, L, Mk, D, forward_only=False):
     emb, temb = rn(B, T, K).bfloat16(), (0.1 * rn(B, T, K)).bfloat16()
     lora, tlora = (0.3 * rn(B, T, 3 * K)).bfloat16(), (0.03 * rn(B, T, 3 * K)).bfloat16()
     ctx = rn(B, Mk, Kc).bfloat16()
-    rope = torch.from_numpy(nro.rope_angles_3d(T, Hh, W, D)).to(dev).reshape(L, 1, 1, D)
+    rope = rope_angles(pkg, dev, T, Hh, W, D).reshape(L, 1, 1, D)
     gemm = lambda rows, k, n: 2.0 * rows * k * n
     flops = {
         "self_attn_projections": 4 * 2 * gemm(B * L, K, K),
@@ -412,12 +419,11 @@ def copy_calibration(dev):
 def bench_norm_rope(args, pkg, dev, desc_txt, B, H, S, D, backward=False):
     """One step = cosmos_norm_rope on x, tx [B, S, H, D] bf16 -> y, ty (heads-first), through the Python host; with
     ``backward`` one step = cosmos_norm_rope_bwd on x, dy -> dx, dweight (x, dy read once, dx written once)."""
-    nro = entry.load_norm_rope_oracle()
     g = torch.Generator(device=dev).manual_seed(0)
     x = torch.randn((B, S, H, D), generator=g, device=dev).to(torch.bfloat16)
     tx = (torch.randn((B, S, H, D), generator=g, device=dev) * 0.1).to(torch.bfloat16)
     w = (1.0 + 0.1 * torch.randn(D, generator=g, device=dev)).float()
-    angles = torch.from_numpy(nro.rope_angles_3d(24, 44, 80, D)).to(dev)   # 24 x 44 x 80 = 84480 tokens
+    angles = rope_angles(pkg, dev, 24, 44, 80, D)   # 24 x 44 x 80 = 84480 tokens
     assert angles.shape[0] == S
     nbytes = 4 * x.numel() * 2 + angles.numel() * 4 + D * 4     # x, tx in; y, ty out; angles; weight
     step = lambda: pkg.norm_rope(x, w, angles, tx, out_layout="bhsd")
@@ -448,7 +454,7 @@ def bench_norm_rope(args, pkg, dev, desc_txt, B, H, S, D, backward=False):
         "data": "synthetic",
         "config": {"workload": desc_txt, "B": B, "S": S, "H": H, "D": D, "bytes_per_call": nbytes},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": achieved / PEAK_HBM_GBS, "traffic": None if backward else MEASURED_TRAFFIC_BYTES.get("nr"),
+                     "frac": achieved / PEAK_HBM_GBS, "traffic": None if backward else MEASURED_TRAFFIC_BYTES["nr"][0], "traffic_source": None if backward else MEASURED_TRAFFIC_BYTES["nr"][1],
                      "kernel": "norm_rope_bwd_kernel<16, bf16> + norm_rope_dweight_kernel" if backward else "norm_rope_kernel<16, tangent, bf16>",
                      "kernel_ms_avg": avg},
     }
@@ -456,6 +462,7 @@ def bench_norm_rope(args, pkg, dev, desc_txt, B, H, S, D, backward=False):
         copy_calibration(dev)
     if not args.no_cpu and not backward:
         # the same step in torch fp32 on the host cores (library rms_norm + rotation under forward AD), on a sample
+        nro = entry.load_norm_rope_oracle()
         rows = 2048
         xs, txs, ws, as_ = x[:, :rows].float().cpu(), tx[:, :rows].float().cpu(), w.cpu().numpy(), angles[:rows].cpu().numpy()
         nro.norm_rope_torch(xs, ws, as_, txs)
@@ -479,6 +486,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="headline workload only: skip the short timings of c2, c4, c5, c3b")
+    ap.add_argument("--extra-steps", type=int, default=5, help="timed steps of each of the extra workloads")
     ap.add_argument("--gemm-ref", action="store_true",
                     help="also time the vendor bf16 GEMM (torch.matmul) at 8192^3 and 16384^3: what dense MFMA work sustains on this box")
     ap.add_argument("--copy-calib", action="store_true",
@@ -495,7 +504,8 @@ def main():
     torch.cuda.set_device(dev)
     desc_txt, B, H, Lq, Lkv, d, tangents, rms, padded = WORKLOADS[args.workload]
     if tangents == "bwd":
-        return bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d)
+        print(json.dumps(bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, steps=args.steps, warmup=args.warmup)), flush=True)
+        return
     if tangents == "e2e":
         return bench_network(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, forward_only=True, text2world=True)
     if tangents == "network_train":
@@ -508,6 +518,59 @@ def main():
         return bench_module(args, pkg, dev, desc_txt, B, H, Lq, d)
     if tangents in ("norm_rope", "norm_rope_bwd"):
         return bench_norm_rope(args, pkg, dev, desc_txt, B, H, Lq, d, backward=tangents == "norm_rope_bwd")
+    result = bench_attention(args, pkg, lib, dev, args.workload, args.steps, args.warmup, full=True)
+    if args.workload == "c3" and not args.no_extra:
+        # the other configurations of the hot path under the same clock, a few steps each (the headline fields above
+        # are not touched): name -> ms per call through the Python host, TFLOP/s and fraction of the bf16 MFMA peak
+        # by the algorithmic FLOP count, the dominant kernel alone
+        extra = {}
+        for name in ("c2", "c4", "c5", "c3b"):
+            torch.cuda.empty_cache()
+            if WORKLOADS[name][6] == "bwd":
+                r = bench_backward(args, pkg, dev, *WORKLOADS[name][:6], steps=args.extra_steps, warmup=2)
+            else:
+                r = bench_attention(args, pkg, lib, dev, name, args.extra_steps, 2, full=False)
+            extra[name] = {"workload": r["config"]["workload"], "ms": r["ms_per_step"], "tflops": r["value"],
+                           "frac": r["value"] / PEAK_BF16_TFLOPS, "kernel_ms": r["roofline"]["kernel_ms_avg"],
+                           "roofline_bound": r["roofline"]["bound"], "roofline_frac": r["roofline"]["frac"], "steps": r["steps"]}
+        result["extra"] = extra
+    print(json.dumps(result), flush=True)
+
+
+def sampled_parity(oracle, tensors, outputs, key_lens, n_blocks=6, seed=0):
+    """128-row blocks (first, last, random; heads drawn over all of them) of the outputs of a call against the fp32 row-block
+    oracle on the CPU.  Returns the largest max-abs / relative-L2 errors over the blocks (O and dO) and the LSE error."""
+    import numpy as np
+
+    q, k, v, tq, tk, tv = tensors
+    o, to, lse = outputs
+    B, H, Lq, _ = q.shape
+    rng = np.random.default_rng(seed)
+    starts = [0, max(Lq - 128, 0)] + [int(x) for x in rng.integers(0, max(Lq - 128, 1), n_blocks - 2)]
+    worst = {"max_abs": 0.0, "rel_l2": 0.0, "lse_max_abs": 0.0}
+    c = lambda x: None if x is None else x.cpu()
+    for i, r0 in enumerate(starts):
+        b, h = i % B, int(rng.integers(0, H))
+        rows = slice(r0, min(r0 + 128, Lq))
+        o_ref, to_ref, lse_ref = oracle.rows_oracle(c(q[b, h, rows]), c(k[b, h]), c(v[b, h]), None if tq is None else c(tq[b, h, rows]),
+                                                    None if tk is None else c(tk[b, h]), None if tv is None else c(tv[b, h]),
+                                                    kv_len=None if key_lens is None else int(key_lens[b]))
+        for got, want in ((o, o_ref), (to, to_ref)):
+            if got is None:
+                continue
+            ma, rl = oracle.error_metrics(got[b, h, rows].float().cpu(), want)
+            worst["max_abs"], worst["rel_l2"] = max(worst["max_abs"], ma), max(worst["rel_l2"], rl)
+        worst["lse_max_abs"] = max(worst["lse_max_abs"], oracle.error_metrics(lse[b, h, rows].cpu(), lse_ref)[0])
+    worst["blocks"] = len(starts)
+    worst["rows_per_block"] = 128
+    worst["within_tolerance"] = bool(worst["max_abs"] <= 2e-2 and worst["rel_l2"] <= 5e-3 and worst["lse_max_abs"] <= 2e-3)
+    return worst
+
+
+def bench_attention(args, pkg, lib, dev, name, steps, warmup, full=True):
+    """One step = pkg.fwd_jvp (re-tiling kernel + attention kernel through the Python host and the C ABI).  ``full``:
+    also the CPU baseline, the parity check of the timed call's own output and the optional calibration legs."""
+    desc_txt, B, H, Lq, Lkv, d, tangents, rms, padded = WORKLOADS[name]
     q, k, v, tq, tk, tv = make_device_inputs(B, H, Lq, Lkv, d, tangents, rms, dev)
     key_lens = None
     mean_len = Lkv
@@ -524,14 +587,15 @@ def main():
     def step():
         return pkg.fwd_jvp(q, k, v, tq, tk, tv, key_lens=key_lens)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         out = step()
     torch.cuda.synchronize()
-    sec = (time.perf_counter() - t0) / args.steps
+    sec = (time.perf_counter() - t0) / steps
+    out_timed = out          # kept for the parity check after all timing
     del out
 
     # dominant kernel alone (the attention kernel and its few-microsecond merge kernel), HIP events on the launch stream
@@ -554,7 +618,7 @@ def main():
     stream = torch.cuda.current_stream().cuda_stream
     ev = lambda: torch.cuda.Event(enable_timing=True)
     pack_ms, run_ms = [], []
-    for i in range(args.warmup + args.steps):
+    for i in range(warmup + steps):
         e0, e1, e2 = ev(), ev(), ev()
         e0.record()
         assert lib.cosmos_attn_pack_kv(ctypes.byref(D), ws.data_ptr(), ws_bytes, stream) == 0
@@ -564,20 +628,37 @@ def main():
         assert lib.cosmos_attn_fwd_jvp(ctypes.byref(D), ws.data_ptr(), ws_bytes, stream) == 0
         e2.record()
         torch.cuda.synchronize()
-        if i >= args.warmup:
+        if i >= warmup:
             pack_ms.append(e0.elapsed_time(e1))
             run_ms.append(e1.elapsed_time(e2) - e0.elapsed_time(e1))
     run_avg = sum(run_ms) / len(run_ms)
     pack_avg = sum(pack_ms) / len(pack_ms)
-    achieved = flops / (run_avg * 1e-3) / 1e12
 
+    what = {"none": "attn fwd", "q": "attn fwd+JVP (tangent on q)", "full": "attn fwd+JVP"}[tangents]
+    where = {"c2": "2B 480p (L=37440)", "c3": "2B 720p (L=84480)", "c4": "14B 720p (H=40, L=84480)",
+             "c5": "2B text cross-attention (Lq=37440, Lkv<=512, key padding)"}[name]
+    traffic, traffic_source = MEASURED_TRAFFIC_BYTES.get(name, _NO_TRAFFIC)
+    # key padding: the FLOP that count are those of the valid keys and of the matmuls that are not identically zero
+    # (the nominal figure -- 6 matmuls over the padded Lkv -- is kept beside it in `config`)
+    flops_value = flops_alg if padded else flops
+    alg_bytes = sum(x.numel() * x.element_size() for x in (q, k, v, tq, tk, tv, o, to, lse) if x is not None)
+    roofline = {"bound": "mfma", "achieved": flops_value / (run_avg * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s"}
+    if padded:
+        # intensity = algorithmic FLOP / algorithmic bytes is below the ridge (peak FLOP/s / peak B/s): HBM-bound
+        roofline = {"bound": "hbm", "achieved": alg_bytes / (run_avg * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "mfma_frac": flops_value / (run_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+    roofline.update({"frac": roofline["achieved"] / roofline["peak"], "traffic": traffic, "traffic_source": traffic_source,
+                     "algorithmic_bytes": alg_bytes,
+                     "kernel": ("attn_fwd_sym_kernel" if tangents == "none" and not padded else "attn_fwd_jvp_kernel") + " (+ attn_combine_kernel)",
+                     "kernel_ms_avg": run_avg, "kernel_ms_min": min(run_ms),
+                     "kernel_ms_median": sorted(run_ms)[len(run_ms) // 2], "pack_kv_kernel_ms_avg": pack_avg})
     result = {
-        "metric": "attn fwd+JVP TFLOP/s & % bf16 MFMA peak @ 2B 720p (L=84480); ms per call",
-        "value": flops / sec / 1e12,
+        "metric": f"{what} TFLOP/s & % bf16 MFMA peak @ {where}; ms per call",
+        "value": flops_value / sec / 1e12,
         "unit": "TFLOP/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": sec * 1e3,
         "higher_is_better": True,
         "scaling": "weak",
@@ -585,27 +666,28 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": desc_txt, "B": B, "H": H, "Lq": Lq, "Lkv": Lkv, "d": d,
-                   "tangents": tangents, "flop_per_call": flops,
-                   "pct_of_bf16_mfma_peak": 100.0 * flops / sec / 1e12 / PEAK_BF16_TFLOPS},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "kernel": ("attn_fwd_sym_kernel" if tangents == "none" else "attn_fwd_jvp_kernel") + " (+ attn_combine_kernel)",
-                     "kernel_ms_avg": run_avg, "kernel_ms_min": min(run_ms),
-                     "kernel_ms_median": sorted(run_ms)[len(run_ms) // 2], "pack_kv_kernel_ms_avg": pack_avg},
+                   "tangents": tangents, "flop_per_call": flops_value,
+                   "pct_of_bf16_mfma_peak": 100.0 * flops_value / sec / 1e12 / PEAK_BF16_TFLOPS},
+        "roofline": roofline,
     }
     if padded:
         result["config"]["mean_key_len"] = mean_len
-        result["config"]["algorithmic_flop_per_call"] = flops_alg
-        result["config"]["algorithmic_tflops"] = flops_alg / sec / 1e12
+        result["config"]["nominal_flop_per_call"] = flops
+        result["config"]["nominal_tflops"] = flops / sec / 1e12
+    if not full:
+        return result
+    # parity of the timed call's own output (the last timed step), all heads in play: sampled 128-row blocks against the
+    # fp32 row-block oracle on the host -- outside the timed region
+    del ws, o, to
+    oracle = entry.load_oracle()
+    result["parity_sampled"] = sampled_parity(oracle, (q, k, v, tq, tk, tv), out_timed, None if key_lens is None else key_lens.cpu().tolist())
     if args.copy_calib:
         copy_calibration(dev)
     if args.gemm_ref:
         result["gemm_ref"] = gemm_reference(dev)
     if not args.no_cpu:
-        del ws, o, to
-        oracle = entry.load_oracle()
         result["cpu_baseline"] = cpu_baseline(oracle, H, Lkv, d, tangents)
-    print(json.dumps(result), flush=True)
+    return result
 
 
 if __name__ == "__main__":

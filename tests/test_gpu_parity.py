@@ -407,7 +407,9 @@ def test_golden_fixtures(pkg, oracle, gpu):
     for name in mg.CASES:
         (q, k, v, tq, tk, tv), kw = mg.case_inputs(oracle, name)
         if q.dtype == torch.float32:
-            continue   # the fp32 plumbing case is the CPU oracle's own; the kernels take 16-bit inputs
+            # the kernels take 16-bit inputs: the fp32 plumbing case runs on its inputs rounded to bf16 and is held to
+            # the same tolerance against the fp32 expectation (the rounding of the inputs is part of the error)
+            q, k, v, tq, tk, tv = (x.to(torch.bfloat16) for x in (q, k, v, tq, tk, tv))
         print("golden", name, flush=True)
         kl = None if kw["key_lens"] is None else torch.tensor(kw["key_lens"], dtype=torch.int32, device=gpu)
         o, to, lse = pkg.attention_with_lse(*(x.to(gpu) for x in (q, k, v, tq, tk, tv)), causal=kw["causal"], sm_scale=kw["sm_scale"], key_lens=kl)
@@ -502,6 +504,27 @@ def test_config3_shape_2b_720p_fwd_jvp(pkg, oracle, gpu):
     print(f" forward-only O vs forward+JVP O: max_abs={ma:.3e} rel_l2={rl:.3e}", flush=True)
     assert ma <= MAX_ABS and rl <= REL_L2
     assert (lse3 - lse).abs().max().item() <= LSE_ABS
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_config1_shape_plumbing_inputs(pkg, oracle, gpu, seed, dtype):
+    """The CPU plumbing configuration (B=1, H=16, L=2048, d=128, six fp32 tensors ~N(0,1)*0.5, scale 1/sqrt(128), no
+    mask) on the HIP path: the kernels take 16-bit inputs, so the fp32 tensors are rounded to the 16-bit type first.
+    Two bars: against torch math SDPA under torch.func.jvp in fp32 on the SAME rounded inputs (the kernel's own error), and
+    against it on the ORIGINAL fp32 inputs (kernel error + the rounding of the inputs), both at the 16-bit tolerance."""
+    q, k, v, tq, tk, tv = oracle.make_inputs((1, 16, 2048, 128), seed=seed, primal_std=0.5, tangent_std=0.5, dtype=torch.float32)
+    half = [x.to(dtype) for x in (q, k, v, tq, tk, tv)]
+    o, to, lse = pkg.attention_with_lse(*(x.to(gpu) for x in half))
+    torch.cuda.synchronize()
+    o_ref, to_ref = oracle.sdpa_jvp_torch(*(x.float() for x in half))
+    _, _, lse_ref = oracle.closed_form(*(x.float() for x in half))
+    check(oracle, "o (rounded inputs)", o, o_ref)
+    check(oracle, "to (rounded inputs)", to, to_ref)
+    assert oracle.error_metrics(lse.cpu(), lse_ref)[0] <= LSE_ABS
+    o32, to32 = oracle.sdpa_jvp_torch(q, k, v, tq, tk, tv)
+    check(oracle, "o (fp32 inputs)", o, o32)
+    check(oracle, "to (fp32 inputs)", to, to32)
 
 
 def test_config2_shape_480p_forward_ragged(pkg, oracle, gpu):
