@@ -20,7 +20,25 @@ __device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
 }
 
+// A value that exists once per 32-lane half of a wavefront, made visible to both halves: afterwards, in every lane l,
+// `lo` is what lane l % 32 held and `hi` what lane 32 + l % 32 held (one v_permlane32_swap, no LDS round trip).  The
+// instruction is written out: given one value for both of its operands, the compiler's builtin treats its two results as
+// equal and drops one of them.  (s_nop: the instruction may not directly follow the VALU write of its operands.)
+__device__ __forceinline__ void both_halves(float x, float& lo, float& hi) {
+    unsigned a = __builtin_bit_cast(unsigned, x), b = a;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    lo = __builtin_bit_cast(float, a);
+    hi = __builtin_bit_cast(float, b);
+}
+
 constexpr int kFragBytes = 1024;   // one MFMA A-operand fragment: 64 lanes x 16 B
+// The running row max that the softmax exponentials refer to is allowed to lag the true one: it moves (and everything
+// summed so far is rescaled) only when some row of the wavefront has a score more than kMaxSlack above it, in log2
+// units, so p = exp2(s c - m) stays below 2^kMaxSlack.  O = sum p v / sum p and LSE = m + log2 sum p hold for any
+// reference m, and 16-bit rounding of p is relative, so nothing is lost; what is gained is that the rescaling pass over
+// the accumulators, which otherwise runs in nearly every one of a sweep's first dozens of steps (in every step of a short
+// sweep), runs about once per sweep.
+constexpr float kMaxSlack = 6.0f;
 #ifndef COSMOS_ATTN_PREFETCH_GROUPS
 #define COSMOS_ATTN_PREFETCH_GROUPS 2   // LDS operand fetches run this many MFMA groups ahead of use
 #endif

@@ -44,9 +44,11 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stddef.h>
+#include <stdlib.h>
 
 #include <mutex>
 #include <set>
+#include <type_traits>
 #include <utility>
 
 #include "cosmos_attn_hip.h"
@@ -139,6 +141,8 @@ struct AttnParams {
     // `splits` key ranges, one workgroup each, which leave unnormalised partial results for attn_combine_kernel.
     // slot = (pair - n_full) * splits + split; block_m = query rows per workgroup (128, or 384 forward only)
     int n_qt, n_full, n_rem, splits;
+    // attn_qstream_kernel: workgroup id = chunk * BH + (batch * H + head); a chunk is q_chunk consecutive query blocks
+    int BH, q_chunk;
     float* part_acc;           // [slot][block_m][d_v] accumulators; with tangents [slot][block_m][2][d_v] (O, T)
     float4* part_stat;         // [slot][block_m]: (running max in log2 units, row sum of P, row sum of H, 0)
 };
@@ -227,14 +231,14 @@ struct ScoreWave {
     // Fold a tile's lane-local score max into the running max.  Returns the factor by which everything accumulated
     // so far must be rescaled before this tile is added (exactly 1 when no row's max moved).
     __device__ __forceinline__ float update_max(float mx) {
-        {   // max with lane ^ 32 (the other half of the same query column): one VALU swap, no LDS round trip
-            const unsigned bits = __builtin_bit_cast(unsigned, mx);
-            const auto sw = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
-            mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+        {   // max with lane ^ 32 (the other half of the same query column)
+            float lo, hi;
+            both_halves(mx, lo, hi);
+            mx = fmaxf(lo, hi);
         }
         const float m_new = fmaxf(m_run, mx * scale_log2);
         float alpha = 1.0f;
-        if (__any(m_new > m_run)) {
+        if (__any(m_new > m_run + kMaxSlack)) {
             alpha = __builtin_amdgcn_exp2f(m_run - m_new);
             l_run *= alpha;
             r_run *= alpha;
@@ -259,7 +263,10 @@ struct ScoreWave {
     // One step: softmax of the tile whose scores are in `x` (already folded into m_run; `alpha` is the rescale
     // factor that goes with it) interleaved with the score MFMAs of the next tile (K part `kpart`) into `xn`.
     // P^T / H^T go to `ph_out`, `alpha` to `alpha_out` (LDS addresses).
-    __device__ __forceinline__ void step(const Scores& x, Scores& xn, const char* kpart, unsigned ph_out, unsigned alpha_out, float alpha) {
+    // `after_chunk(c)` runs right after the MFMAs of d chunk c, the last use of qf[c] / tqf[c] in the step.
+    struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
+    template <class F = NoHook>
+    __device__ __forceinline__ void step(const Scores& x, Scores& xn, const char* kpart, unsigned ph_out, unsigned alpha_out, float alpha, F after_chunk = F()) {
         V8 pf[2], hf[2];
         V8 fa[NC], fb[NC];
         asm volatile("ds_write_b32 %0, %1" ::"v"(alpha_out + 4 * lane), "v"(alpha) : "memory");
@@ -292,6 +299,7 @@ struct ScoreWave {
                     if (k * C::MFMA_PER_C / EPC == 2) softmax_elem(x, pf, hf, c * EPC + k);
                 SCHED_FENCE();
             }
+            after_chunk(c);
         }
         // hand P^T, H^T over (asm stores: a visible LDS store would make the compiler wait for vmcnt(0), i.e. for
         // the direct-to-LDS fills in flight)
@@ -599,6 +607,360 @@ attn_fwd_jvp_kernel(const AttnParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// Short key sequences (text cross-attention: a few hundred keys against tens of thousands of queries).  With 16 key
+// tiles per query block the kernel above spends more time starting and finishing a workgroup (query load, first fills,
+// normalisation, output stores: none of it overlapped with anything) than sweeping the keys.  Here a workgroup keeps
+// going: it serves `q_chunk` consecutive query blocks of one (batch, head) as ONE stream of steps.  The K/V tiles of the
+// head keep circulating through the LDS rings without a gap (the sweep of the next query block starts where the last
+// one ended, modulo the tile count).  Same roles, rings, hand-over and arithmetic as attn_fwd_jvp_kernel; no causal
+// mask, no key-range split.  All three tangent modes (forward only runs here too: at these lengths the fixed costs
+// decide).
+//
+// At these lengths a query block's own memory traffic (Q, dQ in; O, dO out: 128 KB) weighs as much as its key sweep, and
+// the two only overlap if the traffic is spread over the sweep: a block's 64 KB of stores issued in one step queue up
+// in the compute unit's memory pipeline in front of the K/V fills of the following steps and stall them (measured: the
+// stores then cost their full drain time on top of the sweep).  So, except with tangents on k and v (no LDS left):
+//   * an output wavefront normalises a finished block into a private LDS region (whole rows, 16-byte chunks XOR-swizzled
+//     by row so that neither side has bank conflicts) and goes on accumulating the next block;
+//   * the score wavefront of the pair drains that region to memory a few 1 KB stores per step during the next block's
+//     sweep (16-byte stores covering whole rows).  Its vector-memory counter is not the one that tracks the fills, so
+//     nobody ever waits for a store to retire;
+// With tangents on k and v the output wavefronts store from their accumulators right after a block's last accumulation
+// step.  In every mode the score wavefront fetches the next block's Q / dQ rows into the registers of the current ones,
+// d chunk by d chunk, as the block's last score computation lets go of them (no second register set, no copies).
+// For all this a block has at least two steps (a row of at most 32 keys walks a second, fully masked tile).
+template <int DV, int MODE>
+struct StreamStores {
+    static constexpr bool JVP = MODE != MODE_FWD;
+    static constexpr bool TRICKLE = MODE != MODE_JVP_FULL;
+    static constexpr int NT = JVP ? 2 : 1;                            // tensors stored: O (and dO)
+    static constexpr int DVP = DV < 32 ? DV : 32 * ((DV + 31) / 32);   // channels stored (DV = 16: half an accumulator block)
+    static constexpr int CPR = DVP / 8;                  // 16-byte chunks per row
+    static constexpr int ROW_BYTES = DVP * 2;
+    static constexpr int RPS = 64 / CPR;                 // rows one wavefront-wide 16-byte store covers
+    static constexpr int SPT = 32 / RPS;                 // such stores per tensor, wavefront and block
+    static constexpr int NS = NT * SPT;
+    static constexpr int XP_BYTES = TRICKLE ? NT * 32 * ROW_BYTES : 0;   // LDS region per wavefront pair
+    static constexpr int N_DIRECT = (DVP / 8) * NT;      // stores per output wavefront and block when storing from the accumulators
+};
+
+template <typename T, int DQK, int DV, int MODE>
+__global__ void __attribute__((amdgpu_flat_work_group_size(kAttnThreads, kAttnThreads), amdgpu_waves_per_eu(2, 2)))
+attn_qstream_kernel(const AttnParams p) {
+    typedef AttnCfg<DQK, DV, MODE> C;
+    typedef ScoreWave<T, DQK, DV, MODE> SW;
+    typedef OutputWave<T, DQK, DV, MODE> OW;
+    typedef typename VecOf<T>::v8 V8;
+    typedef typename VecOf<T>::v4 V4;
+    constexpr int NC = C::NC, NDB = C::NDB;
+    constexpr bool JVP = C::JVP;
+    constexpr int KP_BYTES = C::KP_BYTES, VP_BYTES = C::VP_BYTES, TILE_BYTES = C::TILE_BYTES;
+    typedef StreamStores<DV, MODE> ST;
+    constexpr bool TRICKLE = ST::TRICKLE;
+    constexpr int STAT_OFF = C::LDS_BYTES;        // [2 query-block parities][inv_l, r / l][4 wavefronts][64 lanes] floats
+    constexpr int XP_OFF = STAT_OFF + 2 * 2 * 4 * 256;   // [4 wavefront pairs] finished blocks on their way out (TRICKLE)
+    // vmcnt immediates (see attn_fwd_jvp_kernel): the newest IN_FLIGHT fills may still be in flight at the top of a
+    // step; when an output wavefront stored a query block from its accumulators in the step before, so may the N_STORES
+    // stores issued behind them (vector memory operations of a wavefront retire in issue order).
+    constexpr int IN_FLIGHT = 2 * C::KP_LOADS + C::VP_LOADS;
+    constexpr int N_STORES = ST::N_DIRECT;
+    static_assert(IN_FLIGHT + N_STORES < 64, "vmcnt is a 6-bit counter");
+    constexpr int WAIT_FILLS = (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14) | 0x0F70;
+    constexpr int WAIT_FILLS_STORES = ((IN_FLIGHT + N_STORES) & 15) | (((IN_FLIGHT + N_STORES) >> 4) << 14) | 0x0F70;
+
+    const int bid = blockIdx.x;
+    const int bh = bid % p.BH, chunk = bid / p.BH, b = bh / p.H, h = bh % p.H;
+    const int qt0 = chunk * p.q_chunk;                                         // first query block of this workgroup
+    const int nq = p.n_qt - qt0 < p.q_chunk ? p.n_qt - qt0 : p.q_chunk;        // query blocks of this workgroup (>= 1)
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const bool score_role = wave < 4;
+    const int qw = wave & 3;
+    const int j = lane & 31, hh = lane >> 5;
+
+    int kv_len = p.Lkv;
+    if (p.key_lens) { const int kl = p.key_lens[b]; kv_len = kl < kv_len ? (kl < 0 ? 0 : kl) : kv_len; }
+    // key tiles per query block: at least two (a finished block drains, and the next block's rows arrive, during the
+    // sweep).  Tiles past the last valid key are fully masked (a row of at most 32 keys walks one such tile, a row
+    // without a single valid key two); past the end of the packed buffer the fills deliver zeros.
+    int n = kv_len > 0 ? (kv_len + kBlockN - 1) / kBlockN : 1;
+    if (n < 2) n = 2;
+    const int n_flat = nq * n;                     // steps of the whole stream: position f = query block f / n, tile f % n
+
+    char* const kring = smem + C::KRING_OFF;
+    char* const vring = smem + C::VRING_OFF;
+    const __amdgpu_buffer_rsrc_t kv_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(p.kv) + (size_t)bh * p.n_tiles * TILE_BYTES, 0, p.n_tiles * TILE_BYTES, 0x00020000);
+    // position f of the stream reads tile (f + shift) mod n: one shift for all query blocks, so the tiles keep arriving
+    // in the same cyclic order across block boundaries and the fills issued ahead of a boundary are the next block's first
+    const int shift = (((bid >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n;
+    auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane((u + shift) % n); };
+    auto wrap_inc = [&](int t) { ++t; return t >= n ? t - n : t; };
+    const int k_run = ((qw * C::KP_LOADS) % C::KP_FR) * kFragBytes, v_run = ((qw * C::VP_LOADS) % C::VP_FR) * kFragBytes;
+    auto make_job = [&](int tk, int ku, int tv, int vu) {
+        LoadJob jb;
+        jb.rsrc = kv_rsrc; jb.lane_off = lane * 16;
+        jb.k_src = tk * TILE_BYTES + k_run; jb.k_dst = kring + (ku % kRingK) * KP_BYTES + k_run;
+        jb.v_src = tv * TILE_BYTES + KP_BYTES + v_run; jb.v_dst = vring + (vu % kRingV) * VP_BYTES + v_run;
+        return jb;
+    };
+    if (!score_role) {   // fill stream, in issue order:  K(0) K(1) K(2) [V(0) K(3)] | step 0: [V(1) K(4)] | step 1: [V(2) K(5)] | ...
+#pragma unroll
+        for (int u = 0; u < 3; ++u) {
+            const LoadJob jb = make_job(tile_at(u), u, 0, 0);
+            issue_part<C::KP_LOADS>(jb.rsrc, jb.k_dst, jb.lane_off, jb.k_src);
+        }
+        issue_group<C>(make_job(tile_at(3), 3, tile_at(0), 0));
+    }
+
+    auto need_mask = [&](int t) { return t * kBlockN + kBlockN > kv_len; };
+    const unsigned ph_base = C::PH_OFF + qw * C::PH_BYTES, alpha_base = C::ALPHA_OFF + qw * 256, stat_base = STAT_OFF + qw * 256;
+    const unsigned xp_base = XP_OFF + qw * ST::XP_BYTES;
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    int t_v = tile_at(1), t_k = tile_at(4);
+
+    if (score_role) {
+        SW w;
+        w.lane = lane;
+        w.scale_log2 = p.scale_log2;
+        w.sm_scale = p.sm_scale;
+        // Q (and dQ) fragments of a query block: B operand of S^T = K Q^T; lane holds Q[row][16 c + 8 hh .. +7] (rows past
+        // Lq read the last row instead: their results are never stored).  Addresses are a wavefront-uniform base (scalar
+        // registers) plus a 32-bit lane offset (the launch code sends only tensors here whose heads span less than 2 GiB):
+        // no 64-bit per-lane pointers live across the steps.
+        const char* const q_head = reinterpret_cast<const char*>(p.q) + ((int64_t)b * p.q_sb + (int64_t)h * p.q_sh) * 2;
+        const char* const tq_head = reinterpret_cast<const char*>(JVP ? p.tq : p.q) + ((int64_t)b * p.q_sb + (int64_t)h * p.q_sh) * 2;
+        auto q_off = [&](int qt) {
+            int row = qt * kBlockM + qw * 32 + j;
+            row = row < p.Lq ? row : p.Lq - 1;
+            return ((unsigned)row * (unsigned)p.q_sl + 8u * hh) * 2u;
+        };
+        {
+            const unsigned off = q_off(qt0);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                w.qf[c] = *reinterpret_cast<const V8*>(q_head + off + 32 * c);
+                if (JVP) w.tqf[c] = *reinterpret_cast<const V8*>(tq_head + off + 32 * c);
+            }
+        }
+        w.m_run = -INFINITY;
+        w.l_run = 0.f;
+        w.r_run = 0.f;
+        // The next block's rows replace the current ones in place: step n-2 of a block computes the block's last scores,
+        // and right after the MFMAs of d chunk c it fetches chunk c of the next block into the same registers; step n-1
+        // (the next block's first scores) then waits chunk by chunk.  That leaves a load one step to arrive, enough from
+        // the L2 but not from memory: step 0 of the block touches every 128-byte line of those rows (4 bytes per lane).
+        constexpr int Q_LINES = (2 * DQK + 127) / 128;   // lines per row (at most 2: lane half hh takes line hh)
+        int warm_q = 0, warm_tq = 0;
+        // A finished block drains during steps 1 .. n-1 of the next one, step n-2 excepted (its stores would sit behind
+        // that step's row fetches in the memory queue and be waited for together with them): max(1, n-2) steps.
+        const int drain_steps = n > 3 ? n - 2 : 1;
+        const int st_per_step = (ST::NS + drain_steps - 1) / drain_steps;
+        // store number i of a query block's results: tensor i / SPT, rows (i % SPT) RPS .. + RPS - 1 of this wavefront's 32;
+        // lane l stores chunk l % CPR of row l / CPR of those
+        const int rr = lane / ST::CPR, ch = lane % ST::CPR;
+        const unsigned x_lane = rr * ST::ROW_BYTES + ((ch ^ (rr & (ST::CPR - 1))) << 4);
+        const unsigned o_lane = ((unsigned)rr * (unsigned)p.o_sl + 8u * ch) * 2u;
+        const int64_t o_head = ((int64_t)b * p.o_sb + (int64_t)h * p.o_sh) * 2;
+        auto drain = [&](int qt, int lo, int hi) {
+            for (int i = lo; i < hi; ++i) {
+                const int t = i / ST::SPT, g = i % ST::SPT;
+                const unsigned sw = ST::RPS < ST::CPR ? ((g * ST::RPS) & (ST::CPR - 1)) << 4 : 0;   // row g RPS + rr has swizzle key (g RPS + rr) mod CPR
+                const V8 val = *reinterpret_cast<const V8*>(smem + xp_base + t * 32 * ST::ROW_BYTES + g * ST::RPS * ST::ROW_BYTES + (x_lane ^ sw));
+                const int r0 = qt * kBlockM + qw * 32 + g * ST::RPS;
+                char* const base = reinterpret_cast<char*>(t ? p.to : p.o) + o_head + (int64_t)r0 * p.o_sl * 2;
+                if (r0 + rr < p.Lq) asm volatile("global_store_dwordx4 %0, %1, %2 nt" ::"v"(o_lane), "v"(val), "s"(base) : "memory");
+            }
+        };
+
+        typename SW::Scores sc0, sc1;
+        __builtin_amdgcn_s_barrier();         // the K part of the first tile is in LDS (the output wavefronts waited for it)
+        asm volatile("" ::: "memory");
+        float alpha = 1.0f;
+        auto fold = [&](typename SW::Scores& x, int t) {
+            if (need_mask(t)) SW::mask_scores(x, t * kBlockN + 4 * hh, kv_len, false, 0);
+            alpha = w.update_max(SW::lane_max(x));
+        };
+        w.scores_plain(sc0, kring);
+        fold(sc0, tile_at(0));
+        int f = 0, qi = 0;                       // position in the stream, and its query block
+        bool more = nq > 1;                      // is there a block after block qi?
+        // Step f = position s_in of block qi's sweep: softmax of the tile at position f (scores in `cur`), scores of position
+        // f+1 into `nxt`, its statistics.  Three kinds, as separate code: steps 0 .. n-3 of a block; step n-2, which refills
+        // the Q / dQ registers; step n-1, which waits for them chunk by chunk and closes the block.  (Apart, so that the
+        // compiler sees every fetch waited for inside the pair of steps that issues it and puts no waits for it -- which
+        // would wait for the drain stores as well -- into the other steps.)
+        typedef std::integral_constant<int, 0> Plain;
+        typedef std::integral_constant<int, 1> Refill;
+        typedef std::integral_constant<int, 2> Last;
+        auto one = [&](auto kind, typename SW::Scores& cur, typename SW::Scores& nxt, int s_in) {
+            constexpr int KIND = decltype(kind)::value;
+            __builtin_amdgcn_s_waitcnt(0xC07F);      // own LDS stores of step f-1 done
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            const unsigned ph_out = lds0 + ph_base + (f & 1) * 4 * C::PH_BYTES, alpha_out = lds0 + alpha_base + (f & 1) * 4 * 256;
+            const char* const kpart = kring + ((f + 1) % kRingK) * KP_BYTES;
+            if (KIND == 0 && more && s_in == 0) {
+                const unsigned off = q_off(qt0 + qi + 1) - 16u * hh + (Q_LINES > 1 ? 128u * hh : 0u);
+                warm_q = *reinterpret_cast<const int*>(q_head + off);
+                if (JVP) warm_tq = *reinterpret_cast<const int*>(tq_head + off);
+            }
+            if (KIND == 1 && more) {
+                const unsigned off = q_off(qt0 + qi + 1);
+                w.step(cur, nxt, kpart, ph_out, alpha_out, alpha, [&](int c) {
+                    w.qf[c] = __builtin_nontemporal_load(reinterpret_cast<const V8*>(q_head + off + 32 * c));
+                    if (JVP) w.tqf[c] = __builtin_nontemporal_load(reinterpret_cast<const V8*>(tq_head + off + 32 * c));
+                });
+            } else {
+                w.step(cur, nxt, kpart, ph_out, alpha_out, alpha);
+            }
+            if (KIND == 2) asm volatile("" ::"v"(warm_q), "v"(warm_tq));   // the touches are done with (keeps their registers theirs until here)
+            if (TRICKLE && KIND != 1 && qi > 0 && s_in > 0) {
+                const int lo = (KIND == 2 ? drain_steps - 1 : s_in - 1) * st_per_step, hi = lo + st_per_step;
+                drain(qt0 + qi - 1, lo, hi < ST::NS ? hi : ST::NS);
+            }
+            if (KIND == 2) {
+                // statistics of the finished block: 1 / l and r / l to the output wavefront, LSE = (m + log2 l) ln 2
+                float l_lo, l_hi, r_lo, r_hi;
+                both_halves(w.l_run, l_lo, l_hi);
+                both_halves(w.r_run, r_lo, r_hi);
+                const float l_tot = l_lo + l_hi, r_tot = r_lo + r_hi;
+                const float inv_l = 1.0f / l_tot;
+                const float r_over_l = r_tot * inv_l;
+                const unsigned sa = lds0 + stat_base + (qi & 1) * 2 * 4 * 256 + 4 * lane;
+                asm volatile("ds_write_b32 %0, %1" ::"v"(sa), "v"(inv_l) : "memory");
+                asm volatile("ds_write_b32 %0, %1 offset:1024" ::"v"(sa), "v"(r_over_l) : "memory");
+                const int row = (qt0 + qi) * kBlockM + qw * 32 + j;
+                if (row < p.Lq && p.lse && hh == 0)
+                    p.lse[(int64_t)bh * p.Lq + row] = (w.m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
+                w.m_run = -INFINITY; w.l_run = 0.f; w.r_run = 0.f;
+            }
+            if (f + 1 < n_flat) fold(nxt, t_v);
+            t_v = wrap_inc(t_v);   // tile at position f + 2
+            ++f;
+        };
+        // sc0 and sc1 swap roles every step; a block always starts and ends with the current scores in sc0 (after an odd
+        // number of steps the scores move back: 32 register copies per block)
+        for (qi = 0; qi < nq; ++qi) {
+            more = qi + 1 < nq;
+            int s_in = 0;
+            for (; s_in + 2 <= n - 2; s_in += 2) {
+                one(Plain(), sc0, sc1, s_in);
+                one(Plain(), sc1, sc0, s_in + 1);
+            }
+            if (s_in < n - 2) {
+                one(Plain(), sc0, sc1, s_in);
+                sc0 = sc1;
+            }
+            one(Refill(), sc0, sc1, n - 2);
+            one(Last(), sc1, sc0, n - 1);
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);      // step n_flat: the output wavefronts accumulate the last tile
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (TRICKLE) {   // the last block: its region was written during the last step
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            drain(qt0 + nq - 1, 0, ST::NS);
+        }
+    } else {
+        OW w;
+        w.lane = lane;
+        auto zero_acc = [&]() {
+#pragma unroll
+            for (int i = 0; i < NDB; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) { w.acc[i][e] = 0.f; if (JVP) w.acct[i][e] = 0.f; }
+            }
+        };
+        zero_acc();
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        int qi = 0, s_in = 0;
+        bool stored = false;                     // did the previous step issue output stores? (wavefront-uniform)
+        // Step f: accumulate the tile at position f-1 (P^T, H^T, alpha written by the score wavefront during step f-1);
+        // if that was the last tile of its query block, normalise the block, send it off and start the next one from zero.
+        for (int f = 0; f <= n_flat; ++f) {
+            if (stored) __builtin_amdgcn_s_waitcnt(WAIT_FILLS_STORES); else __builtin_amdgcn_s_waitcnt(WAIT_FILLS);
+            stored = false;
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            issue_group<C>(make_job(t_k, f + 4, t_v, f + 1));
+            if (f > 0) {
+                w.step(vring + ((f - 1) % kRingV) * VP_BYTES, smem + ph_base + ((f - 1) & 1) * 4 * C::PH_BYTES,
+                       smem + alpha_base + ((f - 1) & 1) * 4 * 256);
+                if (++s_in == n) {
+                    // O = acc / l ; dO = (T - (r / l) acc) / l   (statistics published by the barrier at the top of this step)
+                    const char* st = smem + stat_base + (qi & 1) * 2 * 4 * 256 + 4 * lane;
+                    const float inv_l = *reinterpret_cast<const float*>(st);
+                    const float r_over_l = *reinterpret_cast<const float*>(st + 1024);
+                    const int row0 = (qt0 + qi) * kBlockM + qw * 32;
+                    if constexpr (TRICKLE) {
+                        // accumulator lane (j, hh) holds channels 32 db + 8 g + 4 hh .. +3 of row j: 8 bytes of 16-byte chunk
+                        // 4 db + g, which goes to chunk position (4 db + g) ^ (j mod CPR) of row j of the region
+                        // (the row address is made opaque here so that the chunk addresses are computed on the spot, one XOR
+                        // each, instead of being kept in registers across the whole stream)
+                        unsigned xw = lds0 + xp_base + j * ST::ROW_BYTES + 8 * hh + ((j & (ST::CPR - 1)) << 4);
+                        asm volatile("" : "+v"(xw));
+#pragma unroll
+                        for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+                            for (int g = 0; g < 4; ++g) {
+                                if (32 * db + 8 * g < DV) {
+                                    const unsigned a = xw ^ ((4 * db + g) << 4);
+                                    V4 ov, tov;
+#pragma unroll
+                                    for (int r = 0; r < 4; ++r) {
+                                        ov[r] = (T)(w.acc[db][4 * g + r] * inv_l);
+                                        if (JVP) tov[r] = (T)((w.acct[db][4 * g + r] - r_over_l * w.acc[db][4 * g + r]) * inv_l);
+                                    }
+                                    asm volatile("ds_write_b64 %0, %1" ::"v"(a), "v"(ov) : "memory");
+                                    if (JVP) asm volatile("ds_write_b64 %0, %1 offset:%2" ::"v"(a), "v"(tov), "n"(32 * ST::ROW_BYTES) : "memory");
+                                }
+                            }
+                        }
+                        __builtin_amdgcn_s_waitcnt(0xC07F);   // the region is complete before the next barrier publishes it
+                    } else if (row0 < p.Lq) {           // wavefront-uniform: every wavefront that stores issues all N_STORES stores
+                        const int row = row0 + j;
+                        const int64_t off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)row * p.o_sl;
+                        T* op = reinterpret_cast<T*>(p.o) + off;
+                        T* top = reinterpret_cast<T*>(p.to) + off;
+                        if (row < p.Lq) {
+#pragma unroll
+                            for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+                                for (int g = 0; g < 4; ++g) {
+                                    const int d = 32 * db + 8 * g + 4 * hh;   // registers 4g..4g+3 are 4 consecutive d
+                                    if (32 * db + 8 * g < DV) {
+                                        V4 ov, tov;
+#pragma unroll
+                                        for (int r = 0; r < 4; ++r) {
+                                            ov[r] = (T)(w.acc[db][4 * g + r] * inv_l);
+                                            if (JVP) tov[r] = (T)((w.acct[db][4 * g + r] - r_over_l * w.acc[db][4 * g + r]) * inv_l);
+                                        }
+                                        asm volatile("global_store_dwordx2 %0, %1, off" ::"v"(op + d), "v"(ov) : "memory");
+                                        if (JVP) asm volatile("global_store_dwordx2 %0, %1, off" ::"v"(top + d), "v"(tov) : "memory");
+                                    }
+                                }
+                            }
+                        }
+                        stored = row0 + 32 <= p.Lq;     // all rows live: every store instruction had a live lane
+                    }
+                    zero_acc();
+                    s_in = 0; ++qi;
+                }
+            }
+            t_v = wrap_inc(t_v); t_k = wrap_inc(t_k);
+        }
+        if (TRICKLE) __builtin_amdgcn_s_barrier();   // hands the last block to the score wavefronts
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // drain the (unused) trailing fills before the LDS is released
+    }
+}
+
+#include "attn_qtan_gfx950.h"
+
+// ---------------------------------------------------------------------------------------------------------------
 // Forward only.  Without tangents a wavefront's whole state (Q fragments, one 32 x d_v accumulator, two score sets)
 // fits the 256 registers that two wavefronts per SIMD leave it, and the softmax VALU work per MFMA is three times
 // that of the tangent modes -- too much for one score wavefront per pair.  So all 8 wavefronts do the same thing,
@@ -655,14 +1017,14 @@ struct SymWave {
     }
     // fold the lane-local max of a tile's scores into the running max; returns the rescale factor (1 if no row moved)
     __device__ __forceinline__ float update_max(float mx) {
-        {
-            const unsigned bits = __builtin_bit_cast(unsigned, mx);
-            const auto sw = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
-            mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+        {   // max with lane ^ 32 (the other half of the same query column)
+            float lo, hi;
+            both_halves(mx, lo, hi);
+            mx = fmaxf(lo, hi);
         }
         const float m_new = fmaxf(m_run, mx * scale_log2);
         float alpha = 1.0f;
-        if (__any(m_new > m_run)) {
+        if (__any(m_new > m_run + kMaxSlack)) {
             alpha = __builtin_amdgcn_exp2f(m_run - m_new);
             l_run *= alpha;
             m_run = m_new;
@@ -965,6 +1327,40 @@ attn_kernel_t pick_dqk(int dqk, int dv, int mode) {
 }
 
 
+// the query-streaming kernel is built for equal head dims (what cross-attention in the DiT uses)
+template <typename T, int D>
+attn_kernel_t pick_stream_mode(int mode) {
+    switch (mode) {
+        case MODE_FWD: return attn_qstream_kernel<T, D, D, MODE_FWD>;
+        case MODE_JVP_Q: return nullptr;   // attn_qtan_kernel (pick_stream)
+        default: return attn_qstream_kernel<T, D, D, MODE_JVP_FULL>;
+    }
+}
+template <typename T>
+attn_kernel_t pick_stream(int dqk, int dv, int mode) {
+    if (dqk != dv) return nullptr;
+    if (mode == MODE_JVP_Q) {   // tangent on q only has a kernel of its own
+        switch (dqk) {
+#ifndef COSMOS_ATTN_ONLY_D128
+            case 16: return attn_qtan_kernel<T, 16, 16>;
+            case 32: return attn_qtan_kernel<T, 32, 32>;
+            case 64: return attn_qtan_kernel<T, 64, 64>;
+#endif
+            case 128: return attn_qtan_kernel<T, 128, 128>;
+            default: return nullptr;
+        }
+    }
+    switch (dqk) {
+#ifndef COSMOS_ATTN_ONLY_D128
+        case 16: return pick_stream_mode<T, 16>(mode);
+        case 32: return pick_stream_mode<T, 32>(mode);
+        case 64: return pick_stream_mode<T, 64>(mode);
+#endif
+        case 128: return pick_stream_mode<T, 128>(mode);
+        default: return nullptr;
+    }
+}
+
 int mode_of(const cosmos_attn_desc* d) {
     if (!d->tq && !d->tk && !d->tv) return MODE_FWD;
     if (d->tq && !d->tk && !d->tv) return MODE_JVP_Q;
@@ -1006,6 +1402,36 @@ SplitPlan plan_split(const cosmos_attn_desc* d) {
     if (splits < 2) return s;
     s.n_rem = rem; s.n_full = s.n_pairs - rem; s.splits = splits;
     return s;
+}
+// Short key sequences go to attn_qstream_kernel: query blocks per workgroup (0 = use the other kernels).  Enough
+// workgroups for about six rounds on the chip keep the last round's imbalance small (key lengths may differ per batch
+// row), and at least two blocks per workgroup are needed for the streaming to pay.
+constexpr int kStreamMaxTiles = 64;       // up to 2048 keys
+constexpr int kStreamMaxChunk = 16;
+constexpr int kStreamRounds = 6;
+int stream_chunk_of(const cosmos_attn_desc* d) {
+    if (d->causal || d->d_qk != d->d_v || n_tiles_of(d) > kStreamMaxTiles) return 0;
+    // the kernel addresses q and o inside a head with 32-bit byte offsets
+    if ((int64_t)d->Lq * d->q_stride[2] >= ((int64_t)1 << 30) || (int64_t)d->Lq * d->o_stride[2] >= ((int64_t)1 << 30)) return 0;
+    const int n_qt = (d->Lq + kBlockM - 1) / kBlockM;
+    const int64_t pairs = (int64_t)n_qt * d->B * d->H;
+    int64_t chunk = pairs / (kNumCUs * kStreamRounds);
+    if (const char* e = getenv("COSMOS_ATTN_STREAM_CHUNK")) chunk = atoi(e);
+    if (chunk > kStreamMaxChunk) chunk = kStreamMaxChunk;
+    if (chunk > n_qt) chunk = n_qt;
+    return chunk < 2 ? 0 : (int)chunk;
+}
+// LDS of attn_qstream_kernel: the layout of attn_fwd_jvp_kernel (AttnCfg::LDS_BYTES) + the per-block statistics slots
+size_t stream_lds_bytes_of(const cosmos_attn_desc* d) {
+    const int mode = mode_of(d);
+    const TileGeom g(d->d_qk, d->d_v, mode == MODE_JVP_FULL);
+    const size_t kp = (size_t)g.kpart_frags * kFragBytes, vp = (size_t)(g.tile_frags - g.kpart_frags) * kFragBytes;
+    const size_t ph = (mode == MODE_FWD ? 2 : 4) * kFragBytes;
+    const int dvp = d->d_v < 32 ? d->d_v : 32 * ((d->d_v + 31) / 32);
+    const size_t xp = mode == MODE_JVP_FULL ? 0 : (size_t)4 * (mode == MODE_FWD ? 1 : 2) * 32 * dvp * 2;   // StreamStores::XP_BYTES per wavefront pair
+    if (mode == MODE_JVP_Q)   // QtCfg::LDS_BYTES
+        return kRingK * kp + kRingV * vp + 2 * 4 * 4 * kFragBytes + 2 * 4 * 256 + 2 * 4 * 256 + xp;
+    return kRingK * kp + kRingV * vp + 2 * 4 * ph + 2 * 4 * 256 + 2 * 2 * 4 * 256 + xp;
 }
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 // partial results of the split pairs: fp32 accumulators (O, and T with tangents), then the row statistics
@@ -1107,6 +1533,21 @@ int run_impl(const cosmos_attn_desc* d, const void* workspace, size_t workspace_
     ap.key_lens = d->key_lens;
     ap.H = d->H; ap.Lq = d->Lq; ap.Lkv = d->Lkv; ap.n_tiles = n_tiles_of(d); ap.causal = d->causal;
     ap.sm_scale = d->sm_scale; ap.scale_log2 = d->sm_scale * 1.4426950408889634f;
+    ap.BH = d->B * d->H; ap.q_chunk = 0;
+    ap.n_qt = (d->Lq + kBlockM - 1) / kBlockM; ap.n_full = ap.n_rem = 0; ap.splits = 1;
+    ap.part_acc = nullptr; ap.part_stat = nullptr;
+    if (const int chunk = stream_chunk_of(d)) {   // short key sequences: one workgroup streams `chunk` query blocks
+        attn_kernel_t sfn = d->dtype == COSMOS_ATTN_BF16 ? pick_stream<__bf16>(d->d_qk, d->d_v, mode)
+                                                         : pick_stream<_Float16>(d->d_qk, d->d_v, mode);
+        if (sfn) {
+            const size_t slds = stream_lds_bytes_of(d);
+            if (!allow_lds((const void*)sfn, slds)) return COSMOS_ATTN_LAUNCH_FAILED;
+            ap.q_chunk = chunk;
+            const int64_t sblocks = (int64_t)((ap.n_qt + chunk - 1) / chunk) * ap.BH;
+            hipLaunchKernelGGL(sfn, dim3((unsigned)sblocks), dim3(kAttnThreads), slds, (hipStream_t)stream, ap);
+            return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
+        }
+    }
     const size_t lds = lds_bytes_of(d);
     if (!allow_lds((const void*)fn, lds)) return COSMOS_ATTN_LAUNCH_FAILED;
     SplitPlan sp = plan_split(d);

@@ -219,6 +219,68 @@ def test_single_valid_key(pkg, oracle, gpu):
     assert oracle.error_metrics(lse.cpu(), lse_ref)[0] <= LSE_ABS
 
 
+# ------------------------------------------------------------------ short key sequences: the query-streaming kernels
+# The library sends a call to the streaming kernels only when it has thousands of (query block, head) pairs; the
+# environment variable COSMOS_ATTN_STREAM_CHUNK (query blocks per workgroup, read at every call) forces them on small ones.
+@pytest.mark.parametrize("chunk", [2, 3, 16])
+@pytest.mark.parametrize("tangents", ["q", "none", "full"])
+def test_streaming_kernels_key_tile_counts(pkg, oracle, gpu, monkeypatch, chunk, tangents):
+    monkeypatch.setenv("COSMOS_ATTN_STREAM_CHUNK", str(chunk))
+    for i, Lkv in enumerate([1, 20, 32, 33, 64, 96, 100, 160, 257, 512]):
+        if Lkv == 1 and tangents == "q":
+            continue   # one key: the q-tangent cancels to rounding noise (test_single_valid_key), a relative measure means nothing
+        run_case(pkg, oracle, gpu, (1, 2, 700, 128), (1, 2, Lkv, 128), tangents=tangents, seed=10 * chunk + i)
+
+
+@pytest.mark.parametrize("tangents", ["q", "none", "full"])
+@pytest.mark.parametrize("lens", [[64, 512], [7, 33], [300, 31], [2, 65], [96, 97]])
+def test_streaming_kernels_key_padding(pkg, oracle, gpu, monkeypatch, lens, tangents):
+    monkeypatch.setenv("COSMOS_ATTN_STREAM_CHUNK", "4")
+    Lkv = max(lens) if max(lens) > 100 else 100
+    run_case(pkg, oracle, gpu, (2, 3, 1100, 128), (2, 3, Lkv, 128), key_lens=lens, tangents=tangents, seed=sum(lens))
+
+
+@pytest.mark.parametrize("d", [16, 32, 64])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tangents", ["q", "none", "full"])
+def test_streaming_kernels_head_dims(pkg, oracle, gpu, monkeypatch, d, dtype, tangents):
+    monkeypatch.setenv("COSMOS_ATTN_STREAM_CHUNK", "3")
+    run_case(pkg, oracle, gpu, (1, 2, 650, d), (1, 2, 150, d), tangents=tangents, dtype=dtype, seed=d)
+    run_case(pkg, oracle, gpu, (1, 2, 129, d), (1, 2, 70, d), tangents=tangents, dtype=dtype, seed=d + 1)
+
+
+@pytest.mark.parametrize("tangents", ["q", "none"])
+def test_streaming_kernels_match_the_block_kernels_bitwise_free(pkg, oracle, gpu, monkeypatch, tangents):
+    """Streamed and not streamed: same arithmetic per tile, but the streaming kernels may walk the tiles in another
+    cyclic order and pad a one-tile row with a masked tile, so the results agree to rounding, not bit for bit; both must
+    meet the oracle.  Strided (B, L, H, d) views, one query block per workgroup at the end of the stream (1000 rows, 3 per
+    workgroup)."""
+    q, k, v, tq, _, _ = oracle.make_inputs((2, 2, 1000, 128), (2, 2, 300, 128), seed=5)
+    blhd = lambda x: x.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3).to(gpu)   # (B, H, L, d) view of (B, L, H, d) memory
+    args = (blhd(q), blhd(k), blhd(v), blhd(tq) if tangents == "q" else None)
+    kl = torch.tensor([300, 77], dtype=torch.int32, device=gpu)
+    monkeypatch.setenv("COSMOS_ATTN_STREAM_CHUNK", "1")
+    ref = pkg.attention_with_lse(*args, key_lens=kl)
+    monkeypatch.setenv("COSMOS_ATTN_STREAM_CHUNK", "3")
+    got = pkg.attention_with_lse(*args, key_lens=kl)
+    torch.cuda.synchronize()
+    o_ref, to_ref, lse_ref = oracle.closed_form(q, k, v, tq if tangents == "q" else None, None, None, key_lens=[300, 77])
+    for res in (ref, got):
+        check(oracle, "o", res[0], o_ref)
+        if tangents == "q":
+            check(oracle, "to", res[1], to_ref)
+        assert oracle.error_metrics(res[2].cpu(), lse_ref)[0] <= LSE_ABS
+    assert (got[0].float() - ref[0].float()).abs().max().item() <= 1e-2
+
+
+def test_streaming_kernel_reproducible(pkg, oracle, gpu, monkeypatch):
+    monkeypatch.setenv("COSMOS_ATTN_STREAM_CHUNK", "5")
+    q, k, v, tq, _, _ = oracle.make_inputs((1, 4, 2000, 128), (1, 4, 200, 128), seed=8)
+    a = pkg.attention_with_lse(q.to(gpu), k.to(gpu), v.to(gpu), tq.to(gpu))
+    b = pkg.attention_with_lse(q.to(gpu), k.to(gpu), v.to(gpu), tq.to(gpu))
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+
+
 # ------------------------------------------------------------------ the reference's own test shapes
 @pytest.mark.parametrize("shape", [(1, 2, 1024, 64), (1, 2, 999, 64)])
 @pytest.mark.parametrize("causal", [True, False])
