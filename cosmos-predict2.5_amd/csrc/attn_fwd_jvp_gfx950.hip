@@ -1485,6 +1485,7 @@ COSMOS_ATTN_API const char* cosmos_attn_status_string(int status) {
         case COSMOS_ATTN_UNSUPPORTED: return "unsupported dtype or head dim (bf16/fp16, head dim <= 128)";
         case COSMOS_ATTN_WORKSPACE_TOO_SMALL: return "workspace too small or null";
         case COSMOS_ATTN_LAUNCH_FAILED: return "kernel launch failed";
+        case COSMOS_ATTN_STATIC_SCRATCH_EXCEEDED: return "problem needs more workspace than the library's static scratch array holds (cosmos_attn_static_scratch_bytes); use cosmos_attn_fwd_jvp with a caller-provided workspace";
         default: return "unknown status";
     }
 }
@@ -1586,6 +1587,50 @@ COSMOS_ATTN_API int cosmos_attn_fwd_jvp(const cosmos_attn_desc* d, void* workspa
     if (st != COSMOS_ATTN_OK) return st;
     void* scratch = partial_bytes_of(d) ? (char*)workspace + align256(tiles_bytes_of(d)) : nullptr;
     return run_impl(d, workspace, workspace_bytes, scratch, stream);
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------------------------------------------
+// The same call for callers that cannot allocate (code under graph capture, serving loops, harnesses that forbid it):
+// the workspace (re-tiled K/V image + key-range partial results) is a device array that is part of this library's
+// code object.  Every GPU the library runs on holds its own copy, at its own address, until the process ends; the array's
+// name is only a handle on the host, so its address on the current device is looked up once per device and kept.
+namespace {
+constexpr size_t kStaticScratchBytes = (size_t)COSMOS_ATTN_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};       // device address of `scratch`, per device ordinal (null: not looked up yet)
+std::mutex g_scratch_mu;
+
+// device address of the current device's copy of `scratch` (null on failure)
+void* static_scratch_ptr() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) { (void)hipGetLastError(); return nullptr; }
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) { (void)hipGetLastError(); return nullptr; }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" {
+
+COSMOS_ATTN_API size_t cosmos_attn_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+COSMOS_ATTN_API int cosmos_attn_fwd_jvp_static(const cosmos_attn_desc* d, void* stream) {
+    const int st = validate(d);
+    if (st != COSMOS_ATTN_OK) return st;
+    const size_t need = cosmos_attn_workspace_bytes(d);
+    if (need > kStaticScratchBytes) return COSMOS_ATTN_STATIC_SCRATCH_EXCEEDED;
+    void* const ws = static_scratch_ptr();
+    if (!ws) return COSMOS_ATTN_LAUNCH_FAILED;
+    // nothing in the workspace has to start at zero: the re-tiling kernel writes every byte of the image (padding
+    // included) and every key range writes its whole slot of partial results before the merge kernel reads it
+    return cosmos_attn_fwd_jvp(d, ws, need, stream);
 }
 
 }  // extern "C"

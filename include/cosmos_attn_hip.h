@@ -39,8 +39,12 @@ enum cosmos_attn_status {
     COSMOS_ATTN_BAD_STRIDE = 3,     /* misaligned base or stride (16-byte rows required) */
     COSMOS_ATTN_UNSUPPORTED = 4,    /* dtype / head-dim combination not built */
     COSMOS_ATTN_WORKSPACE_TOO_SMALL = 5,
-    COSMOS_ATTN_LAUNCH_FAILED = 6   /* hipGetLastError() != hipSuccess after a launch */
+    COSMOS_ATTN_LAUNCH_FAILED = 6,  /* hipGetLastError() != hipSuccess after a launch */
+    COSMOS_ATTN_STATIC_SCRATCH_EXCEEDED = 7   /* cosmos_attn_fwd_jvp_static: workspace need > COSMOS_ATTN_STATIC_SCRATCH_BYTES */
 };
+
+/* size of the static device array behind cosmos_attn_fwd_jvp_static (64 MiB) */
+#define COSMOS_ATTN_STATIC_SCRATCH_BYTES (64u << 20)
 
 /*
  * One attention call.  Tensors are [B, H, L, d] addressed through element strides
@@ -96,6 +100,21 @@ COSMOS_ATTN_API size_t cosmos_attn_workspace_bytes(const cosmos_attn_desc *desc)
  * Launches the re-tiling kernel and the attention kernel on `stream`; returns a status code.
  */
 COSMOS_ATTN_API int cosmos_attn_fwd_jvp(const cosmos_attn_desc *desc, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * cosmos_attn_fwd_jvp without a workspace argument and without any allocation: the workspace is a static device array
+ * inside the library (COSMOS_ATTN_STATIC_SCRATCH_BYTES = 64 MiB per GPU, held until the process ends).
+ * No counterpart in the reference.  It is for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The call itself calls no hipMalloc / hipFree and no
+ * allocating library routine; inputs and outputs are the caller's, as in cosmos_attn_fwd_jvp, and results are bitwise
+ * those of cosmos_attn_fwd_jvp.
+ * A problem whose cosmos_attn_workspace_bytes() exceeds the array is refused with COSMOS_ATTN_STATIC_SCRATCH_EXCEEDED
+ * (the text cross-attention of the 2B DiT, B=2 H=16 Lkv=512 d=128, needs 8 MiB; self-attention at L=84480 does not fit).
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or threads)
+ * race on it; calls on one stream are ordered and safe.
+ */
+COSMOS_ATTN_API size_t cosmos_attn_static_scratch_bytes(void);
+COSMOS_ATTN_API int cosmos_attn_fwd_jvp_static(const cosmos_attn_desc *desc, void *stream);
 
 /*
  * The two stages separately, for callers that reuse K/V across calls (e.g. cross-attention
