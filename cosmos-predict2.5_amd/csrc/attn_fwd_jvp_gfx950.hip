@@ -958,8 +958,6 @@ attn_qstream_kernel(const AttnParams p) {
     }
 }
 
-#include "attn_qtan_gfx950.h"
-
 // ---------------------------------------------------------------------------------------------------------------
 // Forward only.  Without tangents a wavefront's whole state (Q fragments, one 32 x d_v accumulator, two score sets)
 // fits the 256 registers that two wavefronts per SIMD leave it, and the softmax VALU work per MFMA is three times
@@ -1332,24 +1330,13 @@ template <typename T, int D>
 attn_kernel_t pick_stream_mode(int mode) {
     switch (mode) {
         case MODE_FWD: return attn_qstream_kernel<T, D, D, MODE_FWD>;
-        case MODE_JVP_Q: return nullptr;   // attn_qtan_kernel (pick_stream)
+        case MODE_JVP_Q: return attn_qstream_kernel<T, D, D, MODE_JVP_Q>;
         default: return attn_qstream_kernel<T, D, D, MODE_JVP_FULL>;
     }
 }
 template <typename T>
 attn_kernel_t pick_stream(int dqk, int dv, int mode) {
     if (dqk != dv) return nullptr;
-    if (mode == MODE_JVP_Q) {   // tangent on q only has a kernel of its own
-        switch (dqk) {
-#ifndef COSMOS_ATTN_ONLY_D128
-            case 16: return attn_qtan_kernel<T, 16, 16>;
-            case 32: return attn_qtan_kernel<T, 32, 32>;
-            case 64: return attn_qtan_kernel<T, 64, 64>;
-#endif
-            case 128: return attn_qtan_kernel<T, 128, 128>;
-            default: return nullptr;
-        }
-    }
     switch (dqk) {
 #ifndef COSMOS_ATTN_ONLY_D128
         case 16: return pick_stream_mode<T, 16>(mode);
@@ -1429,8 +1416,6 @@ size_t stream_lds_bytes_of(const cosmos_attn_desc* d) {
     const size_t ph = (mode == MODE_FWD ? 2 : 4) * kFragBytes;
     const int dvp = d->d_v < 32 ? d->d_v : 32 * ((d->d_v + 31) / 32);
     const size_t xp = mode == MODE_JVP_FULL ? 0 : (size_t)4 * (mode == MODE_FWD ? 1 : 2) * 32 * dvp * 2;   // StreamStores::XP_BYTES per wavefront pair
-    if (mode == MODE_JVP_Q)   // QtCfg::LDS_BYTES
-        return kRingK * kp + kRingV * vp + 2 * 4 * 4 * kFragBytes + 2 * 4 * 256 + 2 * 4 * 256 + xp;
     return kRingK * kp + kRingV * vp + 2 * 4 * ph + 2 * 4 * 256 + 2 * 2 * 4 * 256 + xp;
 }
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
