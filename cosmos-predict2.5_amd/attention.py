@@ -8,11 +8,14 @@ Behaviour kept: cast of q,k,v to ``dtype`` (:110-112), ``q_scale`` (:114-115), `
 unsupported dtypes (:107-108), ``q_lens`` / ``k_lens`` accepted and ignored (:94-95 -- the reference never
 reads them).  The gfx950 kernels are deterministic (no atomics, fixed reduction order), so
 ``deterministic=True`` is honoured instead of raising (:151-154).  fp32 is not built: NotImplementedError.
+``dropout_p`` is accepted and not applied, with one warning: this entry stands where the reference calls Flash
+Attention 3 (:119-127), a call that does not receive ``dropout_p`` either.
 """
 from __future__ import annotations
 
 import contextlib
 import threading
+import warnings
 
 import torch
 
@@ -77,6 +80,9 @@ class _AttentionFn(torch.autograd.Function):
         return t(dq), t(dk), t(dv), None, None
 
 
+_warned_dropout = False
+
+
 def attention(
     q,
     k,
@@ -92,9 +98,17 @@ def attention(
 ):
     supported_dtypes = [torch.bfloat16, torch.float16]
     if dtype not in supported_dtypes:
+        # the reference also lists float32 (served by SDPA's efficient-attention backend, attention.py:145-148); the HIP
+        # kernels compute from 16-bit operands only
         raise NotImplementedError(f"{dtype=} is not supported.")
     if dropout_p != 0.0:
-        raise NotImplementedError("dropout is not supported by the HIP attention kernels")
+        # This entry stands where the reference calls Flash Attention 3 (attention.py:119-127), and that call does not
+        # receive dropout_p either: on that branch the argument has no effect.  Same here, said once.
+        global _warned_dropout
+        if not _warned_dropout:
+            _warned_dropout = True
+            warnings.warn("attention(): dropout_p is not applied by the HIP kernels (as on the reference's Flash Attention 3 "
+                          "branch, which does not forward it)", stacklevel=2)
     del q_lens, k_lens, deterministic
 
     q = q.to(dtype)

@@ -338,6 +338,21 @@ def test_attention_forward_matches_sdpa(pkg, oracle, gpu):
     check(oracle, "attention(causal, fp16)", out, ref)
 
 
+def test_attention_forward_dropout_argument_is_not_applied(pkg, oracle, gpu):
+    """attention(dropout_p=...) behaves as on the reference's Flash Attention 3 branch (attention.py:119-127), which does not
+    forward the argument: same result as without it, and the host says so once."""
+    import warnings
+    q, k, v, _, _, _ = oracle.make_inputs((1, 2, 200, 128), seed=9)
+    bshd = lambda x: x.to(gpu).transpose(1, 2).contiguous()
+    ref = pkg.attention_forward(bshd(q), bshd(k), bshd(v))
+    with warnings.catch_warnings(record=True) as w:
+        warnings.simplefilter("always")
+        out = pkg.attention_forward(bshd(q), bshd(k), bshd(v), dropout_p=0.1)
+        pkg.attention_forward(bshd(q), bshd(k), bshd(v), dropout_p=0.1)
+    assert torch.equal(out, ref)
+    assert sum("dropout_p" in str(x.message) for x in w) <= 1
+
+
 def test_attn_op_protocol(pkg, oracle, gpu):
     """a2a_cp.py:208-219 / minimal_v4_dit.py:252-283: op(q,k,v [B,S,H,D]) -> [B,S,H*D]; cross-attention lengths differ."""
     B, S, H, D, Lc = 2, 200, 4, 128, 77

@@ -445,8 +445,8 @@ def test_python_argument_checks_mirror_reference(pkg):
         pkg.attention_jvp(q, q, q, q.transpose(1, 2).contiguous().transpose(1, 2), q, q)
     with pytest.raises(NotImplementedError):                # attention(): dtype not in the supported list (attention.py:107-108)
         pkg.attention_forward(q.transpose(1, 2), q.transpose(1, 2), q.transpose(1, 2), dtype=torch.float64)
-    with pytest.raises(NotImplementedError):
-        pkg.attention_forward(q.transpose(1, 2), q.transpose(1, 2), q.transpose(1, 2), dropout_p=0.1)
+    with pytest.raises(NotImplementedError):                # float32 is on the reference's list (SDPA, :145-148) but not built here
+        pkg.attention_forward(q.transpose(1, 2), q.transpose(1, 2), q.transpose(1, 2), dtype=torch.float32)
 
 
 def test_attn_op_refuses_multi_gpu_group(pkg):
