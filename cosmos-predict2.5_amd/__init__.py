@@ -12,6 +12,6 @@ from .dit_network import FinalLayer, MinimalV1LVGDiT, MiniTrainDIT, PatchEmbed, 
 from .flash_attention_jvp import attention as attention_jvp
 from .flash_attention_jvp import attention_with_lse
 from .rope_position import VideoRopePosition3DEmb
-from .ops import bwd, fwd_jvp, gated_residual, gelu, ln_modulate, norm_rope, norm_rope_bwd
+from .ops import PackedKV, bwd, fwd_jvp, gated_residual, gelu, ln_modulate, norm_rope, norm_rope_bwd, pack_kv, run_packed
 
-__all__ = ["attention_jvp", "attention_with_lse", "attention_forward", "HipAttnOp", "hip_attention_op", "fwd_jvp", "bwd", "norm_rope", "norm_rope_bwd", "ln_modulate", "gated_residual", "gelu", "Attention", "I2VCrossAttention", "Block", "GPT2FeedForward", "MiniTrainDIT", "MinimalV1LVGDiT", "FinalLayer", "PatchEmbed", "TimestepEmbedding", "Timesteps", "VideoRopePosition3DEmb"]
+__all__ = ["attention_jvp", "attention_with_lse", "attention_forward", "HipAttnOp", "hip_attention_op", "fwd_jvp", "pack_kv", "run_packed", "PackedKV", "bwd", "norm_rope", "norm_rope_bwd", "ln_modulate", "gated_residual", "gelu", "Attention", "I2VCrossAttention", "Block", "GPT2FeedForward", "MiniTrainDIT", "MinimalV1LVGDiT", "FinalLayer", "PatchEmbed", "TimestepEmbedding", "Timesteps", "VideoRopePosition3DEmb"]

@@ -179,6 +179,7 @@ EXPORTS = {
     "cosmos_attn_fwd_jvp": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "cosmos_attn_static_scratch_bytes": (ctypes.c_size_t, []),
     "cosmos_attn_fwd_jvp_static": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p]),
+    "cosmos_attn_packed_bytes": (ctypes.c_size_t, [ctypes.POINTER(AttnDesc)]),
     "cosmos_attn_pack_kv": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "cosmos_attn_run": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "cosmos_attn_bwd_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(AttnBwdDesc)]),

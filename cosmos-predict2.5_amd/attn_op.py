@@ -59,3 +59,11 @@ class HipAttnOp(torch.nn.Module):
         o, to, _ = ops.fwd_jvp(tr(query), tr(key), tr(value), tr(t_query), tr(t_key), tr(t_value),
                                out_layout="blhd", need_lse=False)
         return o.transpose(1, 2).flatten(-2), to.transpose(1, 2).flatten(-2)
+
+    def forward_packed(self, query, packed, t_query=None):
+        """The op against a packed (key, value) pair (``ops.pack_kv``): query ``[B, S, H, D]``; returns ``[B, S, H*D]``, and the
+        tangent along ``t_query`` as well when that is given."""
+        tr = lambda x: None if x is None else x.transpose(1, 2)
+        o, to, _ = ops.run_packed(tr(query), packed, tr(t_query), out_layout="blhd", need_lse=False)
+        o = o.transpose(1, 2).flatten(-2)
+        return o if t_query is None else (o, to.transpose(1, 2).flatten(-2))

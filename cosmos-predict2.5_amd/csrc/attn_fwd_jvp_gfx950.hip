@@ -1480,10 +1480,15 @@ COSMOS_ATTN_API size_t cosmos_attn_workspace_bytes(const cosmos_attn_desc* d) {
     return align256(tiles_bytes_of(d)) + partial_bytes_of(d);
 }
 
+COSMOS_ATTN_API size_t cosmos_attn_packed_bytes(const cosmos_attn_desc* d) {
+    if (validate(d) != COSMOS_ATTN_OK) return 0;
+    return align256(tiles_bytes_of(d));
+}
+
 COSMOS_ATTN_API int cosmos_attn_pack_kv(const cosmos_attn_desc* d, void* workspace, size_t workspace_bytes, void* stream) {
     const int st = validate(d);
     if (st != COSMOS_ATTN_OK) return st;
-    if (!workspace || workspace_bytes < cosmos_attn_workspace_bytes(d) || !aligned16(workspace)) return COSMOS_ATTN_WORKSPACE_TOO_SMALL;
+    if (!workspace || workspace_bytes < align256(tiles_bytes_of(d)) || !aligned16(workspace)) return COSMOS_ATTN_WORKSPACE_TOO_SMALL;
     PackParams pp;
     const bool full = mode_of(d) == MODE_JVP_FULL;
     pp.k = (const uint16_t*)d->k; pp.v = (const uint16_t*)d->v;
@@ -1504,7 +1509,9 @@ namespace {
 int run_impl(const cosmos_attn_desc* d, const void* workspace, size_t workspace_bytes, void* scratch, void* stream) {
     const int st = validate(d);
     if (st != COSMOS_ATTN_OK) return st;
-    if (!workspace || workspace_bytes < cosmos_attn_workspace_bytes(d) || !aligned16(workspace)) return COSMOS_ATTN_WORKSPACE_TOO_SMALL;
+    // the two-stage run never cuts key ranges: it needs the image only
+    const size_t need = scratch ? cosmos_attn_workspace_bytes(d) : align256(tiles_bytes_of(d));
+    if (!workspace || workspace_bytes < need || !aligned16(workspace)) return COSMOS_ATTN_WORKSPACE_TOO_SMALL;
     const int mode = mode_of(d);
     attn_kernel_t fn = d->dtype == COSMOS_ATTN_BF16 ? pick_dqk<__bf16>(d->d_qk, d->d_v, mode)
                                                     : pick_dqk<_Float16>(d->d_qk, d->d_v, mode);

@@ -19,6 +19,7 @@ tangent pass of the distillation recipes is taken under ``no_grad``).
 from __future__ import annotations
 
 import math
+import weakref
 from typing import Optional, Tuple
 
 import torch
@@ -100,6 +101,12 @@ class Attention(nn.Module):
         self.output_proj = nn.Linear(inner_dim, query_dim, bias=False)
         self.output_dropout = nn.Dropout(dropout) if dropout > 1e-4 else nn.Identity()
         self.attn_op = HipAttnOp()
+        # Cross-attention against a context that does not change between calls (the text conditioning over the steps of a
+        # sampler, or over the two passes of a JVP): its projected, normalised and re-tiled keys and values are kept per
+        # context tensor and reused while neither that tensor nor the weights that made them have changed.  Used only where
+        # no graph is recorded (inference and forward mode).  ``cache_context = False`` turns it off.
+        self.cache_context = True
+        self._context_cache = {}
 
         self._query_dim = query_dim
         self._context_dim = context_dim
@@ -143,6 +150,32 @@ class Attention(nn.Module):
             return _NormRopeFn.apply(t, norm.weight, rope, norm.eps), None
         return ops.norm_rope(t, norm.weight, rope, tt, eps=norm.eps, out_layout="bhsd")
 
+    def _packed_context(self, slot: str, context: torch.Tensor, k_proj: nn.Linear, k_norm, v_proj: nn.Linear) -> "ops.PackedKV":
+        """Keys and values of ``context`` (projection, per-head RMSNorm, no rotation), re-tiled for the kernels.  The entry
+        is reused only for the very same tensor object (held by a weak reference, so a new tensor that happens to get the
+        freed one's address is never mistaken for it) at the same version, with weights at the same address and version."""
+        params = (k_proj.weight, k_norm.weight, v_proj.weight)
+        key = (context._version, tuple(context.shape), context.dtype, context.device,
+               tuple((w.data_ptr(), w._version, w.dtype) for w in params))
+        hit = self._context_cache.get(slot) if self.cache_context else None
+        if hit is not None and hit[0]() is context and hit[1] == key:
+            return hit[2]
+        k, _ = self._norm_rope(self._heads(k_proj(context)), k_norm, None)
+        v = self._heads(v_proj(context))
+        packed = ops.pack_kv(k.transpose(1, 2), v.transpose(1, 2))
+        if self.cache_context:
+            self._context_cache[slot] = (weakref.ref(context), key, packed)
+        return packed
+
+    def __getstate__(self):
+        state = self.__dict__.copy()
+        state["_context_cache"] = {}          # weak references and device images are not part of a copy of the module
+        return state
+
+    def _context_is_fixed(self, x: torch.Tensor, context) -> bool:
+        return (context is not None) and isinstance(context, torch.Tensor) and x.is_cuda and not torch.is_grad_enabled() \
+            and isinstance(self.v_norm, nn.Identity)
+
     # ------------------------------------------------------------------ the reference's surface
     def compute_qkv(self, x, context=None, rope_emb=None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         """q, k, v as ``[B, S, H, D]`` (q and k in heads-first memory, ready for the kernels)."""
@@ -161,6 +194,11 @@ class Attention(nn.Module):
     def forward(self, x, context: Optional[torch.Tensor] = None, rope_emb: Optional[torch.Tensor] = None, video_size=None):
         """x: ``[B, Mq, K]`` (or ``[B, T, H, W, K]``); context: ``[B, Mk, Kc]`` or None for self-attention; rope_emb: the
         angles ``[Mq, 1, 1, D]`` (self-attention only).  Returns ``[B, Mq, K]`` in the shape of x."""
+        if self._context_is_fixed(x, context):
+            q, _ = self._norm_rope(self._heads(self.q_proj(x)), self.q_norm, rope_emb)
+            packed = self._packed_context("context", context, self.k_proj, self.k_norm, self.v_proj)
+            out = self.output_dropout(self.output_proj(self.attn_op.forward_packed(q, packed)))
+            return out.reshape(*x.shape[:-1], out.shape[-1])
         q, k, v = self.compute_qkv(x, context, rope_emb=rope_emb)
         out = self.compute_attention(q, k, v, video_size=video_size)
         return out.reshape(*x.shape[:-1], out.shape[-1])
@@ -178,6 +216,13 @@ class Attention(nn.Module):
             raise NotImplementedError("forward_jvp with active dropout")
         xs = self._stack(x, tx)
         q, tq = self._apply_stacked(self.q_proj, xs, True)
+        if tcontext is None and self._context_is_fixed(x, context):
+            q, tq = self._norm_rope(self._heads(q), self.q_norm, rope_emb, self._heads(tq))
+            packed = self._packed_context("context", context, self.k_proj, self.k_norm, self.v_proj)
+            o, to = self.attn_op.forward_packed(q, packed, tq)
+            out, tout = self._apply_stacked(self.output_proj, self._stack(o, to), True)
+            shape = (*x.shape[:-1], out.shape[-1])
+            return out.reshape(shape), tout.reshape(shape)
         if context is None:
             k, tk = self._apply_stacked(self.k_proj, xs, True)
             v, tv = self._apply_stacked(self.v_proj, xs, True)
@@ -228,6 +273,13 @@ class I2VCrossAttention(Attention):
 
     def forward(self, x, context=None, rope_emb=None, video_size=None):
         del video_size
+        if x.is_cuda and not torch.is_grad_enabled():
+            text_context, img_context = context
+            q, _ = self._norm_rope(self._heads(self.q_proj(x)), self.q_norm, rope_emb)
+            result = self.attn_op.forward_packed(q, self._packed_context("text", text_context, self.k_proj, self.k_norm, self.v_proj))
+            result_img = self.attn_op.forward_packed(q, self._packed_context("image", img_context, self.k_img, self.k_img_norm, self.v_img))
+            out = self.output_dropout(self.output_proj(result + result_img))
+            return out.reshape(*x.shape[:-1], out.shape[-1])
         q, k, v, k_img, v_img = self.compute_qkv(x, context, rope_emb)
         out = self.compute_attention(q, k, v, k_img, v_img)
         return out.reshape(*x.shape[:-1], out.shape[-1])
@@ -241,11 +293,15 @@ class I2VCrossAttention(Attention):
         h = self._heads
         q, tq = self._apply_stacked(self.q_proj, self._stack(x, tx), True)
         q, tq = self._norm_rope(h(q), self.q_norm, rope_emb, h(tq))
-        k, _ = self._norm_rope(h(self.k_proj(text_context)), self.k_norm, rope_emb)
-        k_img, _ = self._norm_rope(h(self.k_img(img_context)), self.k_img_norm, None)
-        v, v_img = h(self.v_proj(text_context)), h(self.v_img(img_context))
-        o, to = self.attn_op.forward_jvp(q, k, v, tq)
-        o2, to2 = self.attn_op.forward_jvp(q, k_img, v_img, tq)
+        if x.is_cuda:
+            o, to = self.attn_op.forward_packed(q, self._packed_context("text", text_context, self.k_proj, self.k_norm, self.v_proj), tq)
+            o2, to2 = self.attn_op.forward_packed(q, self._packed_context("image", img_context, self.k_img, self.k_img_norm, self.v_img), tq)
+        else:
+            k, _ = self._norm_rope(h(self.k_proj(text_context)), self.k_norm, rope_emb)
+            k_img, _ = self._norm_rope(h(self.k_img(img_context)), self.k_img_norm, None)
+            v, v_img = h(self.v_proj(text_context)), h(self.v_img(img_context))
+            o, to = self.attn_op.forward_jvp(q, k, v, tq)
+            o2, to2 = self.attn_op.forward_jvp(q, k_img, v_img, tq)
         o.add_(o2)
         to.add_(to2)
         out, tout = self._apply_stacked(self.output_proj, self._stack(o, to), True)

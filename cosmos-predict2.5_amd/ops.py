@@ -41,6 +41,22 @@ def _strides3(x: torch.Tensor):
     return (ctypes.c_int64 * 3)(x.stride(0), x.stride(1), x.stride(2))
 
 
+def _alloc_outputs(B, H, Lq, d_v, q, have_tangent, out_layout, need_lse):
+    if out_layout == "bhld":
+        o = torch.empty((B, H, Lq, d_v), device=q.device, dtype=q.dtype)
+        to = torch.empty_like(o) if have_tangent else None
+    elif out_layout == "blhd" and have_tangent:
+        # o and to as the two halves of one buffer: a following linear layer maps both in one GEMM without a copy
+        both = torch.empty((2, B, Lq, H, d_v), device=q.device, dtype=q.dtype)
+        o, to = both[0].transpose(1, 2), both[1].transpose(1, 2)
+    elif out_layout == "blhd":
+        o, to = torch.empty((B, Lq, H, d_v), device=q.device, dtype=q.dtype).transpose(1, 2), None
+    else:
+        raise ValueError(f"out_layout={out_layout!r}")
+    lse = torch.empty((B, H, Lq), device=q.device, dtype=torch.float32) if need_lse else None
+    return o, to, lse
+
+
 def fwd_jvp(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -93,18 +109,7 @@ def fwd_jvp(
     if sm_scale is None:
         sm_scale = d_qk ** (-0.5)
 
-    if out_layout == "bhld":
-        o = torch.empty((B, H, Lq, d_v), device=q.device, dtype=q.dtype)
-        to = torch.empty_like(o) if have_tangent else None
-    elif out_layout == "blhd" and have_tangent:
-        # o and to as the two halves of one buffer: a following linear layer maps both in one GEMM without a copy
-        both = torch.empty((2, B, Lq, H, d_v), device=q.device, dtype=q.dtype)
-        o, to = both[0].transpose(1, 2), both[1].transpose(1, 2)
-    elif out_layout == "blhd":
-        o, to = torch.empty((B, Lq, H, d_v), device=q.device, dtype=q.dtype).transpose(1, 2), None
-    else:
-        raise ValueError(f"out_layout={out_layout!r}")
-    lse = torch.empty((B, H, Lq), device=q.device, dtype=torch.float32) if need_lse else None
+    o, to, lse = _alloc_outputs(B, H, Lq, d_v, q, have_tangent, out_layout, need_lse)
 
     if key_lens is not None:
         assert not causal, "key_lens with causal is not supported"
@@ -139,6 +144,100 @@ def fwd_jvp(
     _lib.raise_for_status(status)
     # workspace / converted inputs are freed to torch's caching allocator here; it is stream-ordered on
     # the launch stream, so reuse by later work on this stream is safe.
+    return o, to, lse
+
+
+class PackedKV:
+    """The re-tiled image of one (k, v) pair (no tangents), made by :func:`pack_kv` and consumed by :func:`run_packed`:
+    for keys and values that stay the same over many calls (the text context of the DiT's cross-attention)."""
+
+    __slots__ = ("image", "B", "H", "Lkv", "d_qk", "d_v", "dtype", "device")
+
+    def __init__(self, image, B, H, Lkv, d_qk, d_v, dtype, device):
+        self.image, self.B, self.H, self.Lkv, self.d_qk, self.d_v, self.dtype, self.device = image, B, H, Lkv, d_qk, d_v, dtype, device
+
+
+def _packed_desc(B, H, Lq, Lkv, d_qk, d_v, dtype, sm_scale):
+    desc = _lib.AttnDesc()
+    desc.abi_version = _lib.ABI_VERSION
+    desc.dtype = _DTYPES[dtype]
+    desc.B, desc.H, desc.Lq, desc.Lkv, desc.d_qk, desc.d_v = B, H, Lq, Lkv, d_qk, d_v
+    desc.causal = 0
+    desc.sm_scale = float(sm_scale)
+    desc.tk = desc.tv = None
+    return desc
+
+
+def pack_kv(k: torch.Tensor, v: torch.Tensor) -> PackedKV:
+    """Re-tile k, v (``[B, H, Lkv, d]`` views) once (``cosmos_attn_pack_kv``)."""
+    assert k.dim() == 4 and v.dim() == 4 and k.shape[:-1] == v.shape[:-1]
+    B, H, Lkv, d_qk = k.shape
+    d_v = v.shape[-1]
+    assert d_qk in REFERENCE_HEAD_DIMS and d_v in REFERENCE_HEAD_DIMS
+    if d_qk not in SUPPORTED_HEAD_DIMS or d_v not in SUPPORTED_HEAD_DIMS:
+        raise NotImplementedError(f"head dims ({d_qk}, {d_v}): the HIP kernels are built for {SUPPORTED_HEAD_DIMS}")
+    if not k.is_cuda:
+        raise RuntimeError("cosmos attention (HIP) needs tensors on a GPU; there is no CPU path")
+    if k.dtype not in _DTYPES:
+        raise NotImplementedError(f"dtype={k.dtype} is not supported (bf16 / fp16)")
+    assert v.dtype == k.dtype and v.device == k.device
+    k, _ = _prep_pair(k, None)
+    v, _ = _prep_pair(v, None)
+    desc = _packed_desc(B, H, 1, Lkv, d_qk, d_v, k.dtype, 1.0)
+    desc.k, desc.v = k.data_ptr(), v.data_ptr()
+    desc.k_stride, desc.v_stride = _strides3(k), _strides3(v)
+    # pack_kv does not touch q / o: any valid addresses and strides pass the descriptor checks
+    desc.q, desc.o, desc.tq, desc.to, desc.lse, desc.key_lens = k.data_ptr(), k.data_ptr(), None, None, None, None
+    desc.q_stride, desc.o_stride = _strides3(k), _strides3(k)
+    lib = _lib.load_library()
+    with torch.cuda.device(k.device):
+        nbytes = lib.cosmos_attn_packed_bytes(ctypes.byref(desc))
+        if nbytes == 0:
+            _lib.raise_for_status(lib.cosmos_attn_pack_kv(ctypes.byref(desc), None, 0, None) or _lib.ST_BAD_ARG)
+        image = torch.empty(nbytes, device=k.device, dtype=torch.uint8)
+        status = lib.cosmos_attn_pack_kv(ctypes.byref(desc), image.data_ptr(), nbytes, torch.cuda.current_stream(k.device).cuda_stream)
+    _lib.raise_for_status(status)
+    return PackedKV(image, B, H, Lkv, d_qk, d_v, k.dtype, k.device)
+
+
+def run_packed(
+    q: torch.Tensor,
+    packed: PackedKV,
+    tq: Optional[torch.Tensor] = None,
+    sm_scale: Optional[float] = None,
+    key_lens: Optional[torch.Tensor] = None,
+    out_layout: str = "bhld",
+    need_lse: bool = True,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """:func:`fwd_jvp` (forward only, or tangent on q) against a packed (k, v): ``cosmos_attn_run``.  Same results, bit for bit,
+    as the one-call form whenever that one does not cut key ranges (it never does with ``key_lens``)."""
+    assert q.dim() == 4
+    B, H, Lq, d_qk = q.shape
+    assert (B, H, d_qk) == (packed.B, packed.H, packed.d_qk) and q.dtype == packed.dtype and q.device == packed.device
+    if tq is not None:
+        assert tq.shape == q.shape and tq.dtype == q.dtype and tq.device == q.device
+    q, tq = _prep_pair(q, tq)
+    d_v = packed.d_v
+    if sm_scale is None:
+        sm_scale = d_qk ** (-0.5)
+    o, to, lse = _alloc_outputs(B, H, Lq, d_v, q, tq is not None, out_layout, need_lse)
+    if key_lens is not None:
+        key_lens = key_lens.to(device=q.device, dtype=torch.int32).contiguous()
+        assert key_lens.shape == (B,)
+    desc = _packed_desc(B, H, Lq, packed.Lkv, d_qk, d_v, q.dtype, sm_scale)
+    desc.q, desc.tq = q.data_ptr(), (tq.data_ptr() if tq is not None else None)
+    desc.k = desc.v = packed.image.data_ptr()          # only tested for NULL by cosmos_attn_run
+    desc.q_stride = _strides3(q)
+    desc.k_stride = desc.v_stride = (ctypes.c_int64 * 3)(packed.H * packed.Lkv * 8, packed.Lkv * 8, 8)
+    desc.o, desc.to = o.data_ptr(), (to.data_ptr() if to is not None else None)
+    desc.o_stride = _strides3(o)
+    desc.lse = lse.data_ptr() if lse is not None else None
+    desc.key_lens = key_lens.data_ptr() if key_lens is not None else None
+    lib = _lib.load_library()
+    with torch.cuda.device(q.device):
+        status = lib.cosmos_attn_run(ctypes.byref(desc), packed.image.data_ptr(), packed.image.numel(),
+                                     torch.cuda.current_stream(q.device).cuda_stream)
+    _lib.raise_for_status(status)
     return o, to, lse
 
 

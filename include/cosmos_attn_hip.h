@@ -119,9 +119,13 @@ COSMOS_ATTN_API int cosmos_attn_fwd_jvp_static(const cosmos_attn_desc *desc, voi
 /*
  * The two stages separately, for callers that reuse K/V across calls (e.g. cross-attention
  * against a fixed text context, JVP with several tangent directions on q only) and for profiling.
+ *   cosmos_attn_packed_bytes : bytes of the re-tiled image alone (depends on B, H, Lkv, the head dims and on whether
+ *                              k and v carry tangents; not on q): what the two calls below need as `workspace_bytes`
  *   cosmos_attn_pack_kv : k,v(,tk,tv) -> workspace
  *   cosmos_attn_run     : q(,tq), workspace -> o(,to), lse     (desc->k/v/tk/tv are only tested for NULL)
+ * An image packed without tangents serves forward-only runs and runs with a tangent on q alike.
  */
+COSMOS_ATTN_API size_t cosmos_attn_packed_bytes(const cosmos_attn_desc *desc);
 COSMOS_ATTN_API int cosmos_attn_pack_kv(const cosmos_attn_desc *desc, void *workspace, size_t workspace_bytes, void *stream);
 COSMOS_ATTN_API int cosmos_attn_run(const cosmos_attn_desc *desc, const void *workspace, size_t workspace_bytes, void *stream);
 

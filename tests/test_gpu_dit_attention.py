@@ -143,3 +143,56 @@ def test_reference_self_attention_procedure(pkg, gpu, dtype):
         z = (q @ k.transpose(-2, -1)).softmax(dim=-1) @ v
         z_B_S_Q = z.permute(0, 2, 1, 3).reshape(batch_size, sequence_length, n_heads * head_dim) @ attn.output_proj.weight.float().T
     torch.testing.assert_close(y_B_S_Q.float(), z_B_S_Q, atol=5e-3, rtol=5e-3)
+
+
+def test_fixed_context_is_packed_once_and_reused(pkg, gpu, monkeypatch):
+    """Cross-attention against a context tensor that stays the same: its keys / values are projected, normalised and re-tiled
+    on the first call only; later calls (forward and forward mode) reuse the image and give the same bits as a module with the
+    cache turned off.  A change of the context (in place, or another tensor) or of a weight makes a new image."""
+    import copy
+    m = build(pkg, gpu, 256, 96, 2, 128, torch.bfloat16, seed=3)
+    ref = copy.deepcopy(m)          # the cache is not part of a copy
+    ref.cache_context = False
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(2, 300, 256, generator=g).to(gpu, torch.bfloat16)
+    tx = (torch.randn(2, 300, 256, generator=g) * 0.3).to(gpu, torch.bfloat16)
+    context = torch.randn(2, 48, 96, generator=g).to(gpu, torch.bfloat16)
+    calls = []
+    real_pack = pkg.ops.pack_kv
+    monkeypatch.setattr(pkg.ops, "pack_kv", lambda k, v: (calls.append(1), real_pack(k, v))[1])
+
+    def both(mod, ctx):
+        with torch.no_grad():
+            out = mod(x, ctx)
+        out2, tout = mod.forward_jvp(x, tx, ctx)
+        return out, out2, tout
+
+    a = both(m, context)
+    assert len(calls) == 1                                   # forward packed it, forward mode reused it
+    b = both(m, context)
+    assert len(calls) == 1
+    r = both(ref, context)
+    assert len(calls) == 3                                   # cache off: every call packs
+    for x1, x2, x3 in zip(a, b, r):
+        assert torch.equal(x1, x2) and torch.equal(x1, x3)
+    assert torch.equal(a[0], a[1])
+    context.mul_(0.5)                                        # same tensor, new contents
+    c = both(m, context)
+    assert len(calls) == 4 and not torch.equal(c[0], a[0])
+    assert all(torch.equal(u, w) for u, w in zip(c, both(ref, context)))
+    n = len(calls)
+    other = context.clone()                                  # another tensor with the same contents
+    d = both(m, other)
+    assert len(calls) == n + 1 and all(torch.equal(u, w) for u, w in zip(c, d))
+    with torch.no_grad():
+        m.k_proj.weight.mul_(1.5)
+        ref.k_proj.weight.mul_(1.5)
+    n = len(calls)
+    e = both(m, other)
+    assert len(calls) == n + 1 and not torch.equal(e[0], d[0])
+    assert all(torch.equal(u, w) for u, w in zip(e, both(ref, other)))
+    # with a graph being recorded the module does not use the cache (k, v must stay in the graph)
+    n = len(calls)
+    xg = x.clone().requires_grad_(True)
+    m(xg, other).float().sum().backward()
+    assert len(calls) == n and xg.grad is not None

@@ -420,7 +420,10 @@ def test_c_abi_two_stage_equals_one_call(pkg, oracle, gpu):
     torch.cuda.synchronize()
     o2_ref, _, _ = pkg.fwd_jvp(q2, k, v, tq)
     assert torch.equal(o, o2_ref)
-    assert lib.cosmos_attn_run(ctypes.byref(D), ws.data_ptr(), n - 1, st) == L.ST_WORKSPACE
+    npk = lib.cosmos_attn_packed_bytes(ctypes.byref(D))      # the two-stage calls need the image only
+    assert 0 < npk <= n
+    assert lib.cosmos_attn_run(ctypes.byref(D), ws.data_ptr(), npk, st) == 0
+    assert lib.cosmos_attn_run(ctypes.byref(D), ws.data_ptr(), npk - 1, st) == L.ST_WORKSPACE
 
 
 def test_hip_graph_capture_and_replay(pkg, oracle, gpu):
