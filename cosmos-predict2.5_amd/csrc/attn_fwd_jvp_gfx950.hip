@@ -958,6 +958,8 @@ attn_qstream_kernel(const AttnParams p) {
     }
 }
 
+#include "attn_wide_gfx950.h"
+
 // ---------------------------------------------------------------------------------------------------------------
 // Forward only.  Without tangents a wavefront's whole state (Q fragments, one 32 x d_v accumulator, two score sets)
 // fits the 256 registers that two wavefronts per SIMD leave it, and the softmax VALU work per MFMA is three times
@@ -1374,6 +1376,8 @@ size_t tiles_bytes_of(const cosmos_attn_desc* d) { return (size_t)d->B * d->H * 
 
 // How the (query block, head) pairs are dealt out (see choose_splits): the pairs of a partly filled last round of
 // workgroups are cut along the keys, and a small second kernel merges the ranges.
+// a head dim of 256 goes to attn_wide_kernel
+bool is_wide(const cosmos_attn_desc* d) { return d->d_qk == 256 || d->d_v == 256; }
 struct SplitPlan { int block_m, n_qt, n_pairs, n_full, n_rem, splits; };
 SplitPlan plan_split(const cosmos_attn_desc* d) {
     SplitPlan s;
@@ -1382,7 +1386,7 @@ SplitPlan plan_split(const cosmos_attn_desc* d) {
     s.n_qt = (d->Lq + s.block_m - 1) / s.block_m;
     s.n_pairs = s.n_qt * d->B * d->H;
     s.n_rem = 0; s.splits = 1; s.n_full = s.n_pairs;
-    if (d->causal || d->key_lens) return s;          // key ranges of equal work only
+    if (d->causal || d->key_lens || is_wide(d)) return s;          // key ranges of equal work only; not for head dim 256
     const int rem = s.n_pairs % kNumCUs;
     const int n_steps = fwd ? (n_tiles_of(d) + 1) / 2 : n_tiles_of(d);   // barrier steps: 64 keys forward only, 32 with tangents
     const int splits = choose_splits(rem, n_steps);
@@ -1439,8 +1443,7 @@ int validate(const cosmos_attn_desc* d) {
     if (mode < 0) return COSMOS_ATTN_BAD_ARG;          // tangents must be: none, q only, or all three
     if (mode != MODE_FWD && !d->to) return COSMOS_ATTN_BAD_ARG;
     if (d->dtype != COSMOS_ATTN_BF16 && d->dtype != COSMOS_ATTN_FP16) return COSMOS_ATTN_UNSUPPORTED;
-    if (d->d_qk == 256 || d->d_v == 256) return COSMOS_ATTN_UNSUPPORTED;
-    if (!head_dim_ok(d->d_qk) || !head_dim_ok(d->d_v)) return COSMOS_ATTN_BAD_SHAPE;
+    if (!(head_dim_ok(d->d_qk) || d->d_qk == 256) || !(head_dim_ok(d->d_v) || d->d_v == 256)) return COSMOS_ATTN_BAD_SHAPE;
     if (d->causal && d->Lq != d->Lkv) return COSMOS_ATTN_BAD_SHAPE;
     if (d->causal && d->key_lens) return COSMOS_ATTN_BAD_ARG;
     if (!aligned16(d->q) || !aligned16(d->k) || !aligned16(d->v) || !aligned16(d->o)) return COSMOS_ATTN_BAD_STRIDE;
@@ -1465,9 +1468,9 @@ COSMOS_ATTN_API const char* cosmos_attn_status_string(int status) {
     switch (status) {
         case COSMOS_ATTN_OK: return "ok";
         case COSMOS_ATTN_BAD_ARG: return "bad argument (null pointer, non-positive size, ABI version, or tangent set other than none / q only / q,k,v)";
-        case COSMOS_ATTN_BAD_SHAPE: return "bad shape (head dims must be in {16,32,64,128}; causal needs Lq == Lkv)";
+        case COSMOS_ATTN_BAD_SHAPE: return "bad shape (head dims must be in {16,32,64,128,256}; causal needs Lq == Lkv)";
         case COSMOS_ATTN_BAD_STRIDE: return "bad stride or alignment (16-byte aligned bases, strides multiple of 8 elements, innermost stride 1)";
-        case COSMOS_ATTN_UNSUPPORTED: return "unsupported dtype or head dim (bf16/fp16, head dim <= 128)";
+        case COSMOS_ATTN_UNSUPPORTED: return "unsupported dtype or head dim (bf16/fp16; backward and RMSNorm + RoPE: head dim <= 128)";
         case COSMOS_ATTN_WORKSPACE_TOO_SMALL: return "workspace too small or null";
         case COSMOS_ATTN_LAUNCH_FAILED: return "kernel launch failed";
         case COSMOS_ATTN_STATIC_SCRATCH_EXCEEDED: return "problem needs more workspace than the library's static scratch array holds (cosmos_attn_static_scratch_bytes); use cosmos_attn_fwd_jvp with a caller-provided workspace";
@@ -1504,6 +1507,33 @@ COSMOS_ATTN_API int cosmos_attn_pack_kv(const cosmos_attn_desc* d, void* workspa
 }  // extern "C"
 
 namespace {
+typedef void (*wide_kernel_t)(const AttnParams, int, int);
+template <typename T>
+wide_kernel_t pick_wide(int mode) {
+    switch (mode) {
+        case MODE_FWD: return attn_wide_kernel<T, MODE_FWD>;
+        case MODE_JVP_Q: return attn_wide_kernel<T, MODE_JVP_Q>;
+        default: return attn_wide_kernel<T, MODE_JVP_FULL>;
+    }
+}
+int run_wide(const cosmos_attn_desc* d, const void* workspace, void* stream) {
+    const int mode = mode_of(d);
+    AttnParams ap = {};
+    ap.q = d->q; ap.tq = d->tq;
+    ap.q_sb = d->q_stride[0]; ap.q_sh = d->q_stride[1]; ap.q_sl = d->q_stride[2];
+    ap.o = d->o; ap.to = d->to;
+    ap.o_sb = d->o_stride[0]; ap.o_sh = d->o_stride[1]; ap.o_sl = d->o_stride[2];
+    ap.lse = d->lse;
+    ap.kv = (const char*)workspace;
+    ap.key_lens = d->key_lens;
+    ap.H = d->H; ap.Lq = d->Lq; ap.Lkv = d->Lkv; ap.n_tiles = n_tiles_of(d); ap.causal = d->causal;
+    ap.sm_scale = d->sm_scale; ap.scale_log2 = d->sm_scale * 1.4426950408889634f;
+    const int64_t blocks = (int64_t)((d->Lq + 31) / 32) * d->B * d->H;
+    if (blocks > ((int64_t)1 << 31) - 1) return COSMOS_ATTN_BAD_SHAPE;
+    wide_kernel_t fn = d->dtype == COSMOS_ATTN_BF16 ? pick_wide<__bf16>(mode) : pick_wide<_Float16>(mode);
+    hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3(64 * kWideWaves), 0, (hipStream_t)stream, ap, (int)d->d_qk, (int)d->d_v);
+    return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
+}
 // `scratch`: where key-range partial results may go (null: never split).  cosmos_attn_run only reads its workspace, so
 // that several runs may share one re-tiled K/V image; the one-call entry point owns the workspace and passes its tail.
 int run_impl(const cosmos_attn_desc* d, const void* workspace, size_t workspace_bytes, void* scratch, void* stream) {
@@ -1513,6 +1543,7 @@ int run_impl(const cosmos_attn_desc* d, const void* workspace, size_t workspace_
     const size_t need = scratch ? cosmos_attn_workspace_bytes(d) : align256(tiles_bytes_of(d));
     if (!workspace || workspace_bytes < need || !aligned16(workspace)) return COSMOS_ATTN_WORKSPACE_TOO_SMALL;
     const int mode = mode_of(d);
+    if (is_wide(d)) return run_wide(d, workspace, stream);
     attn_kernel_t fn = d->dtype == COSMOS_ATTN_BF16 ? pick_dqk<__bf16>(d->d_qk, d->d_v, mode)
                                                     : pick_dqk<_Float16>(d->d_qk, d->d_v, mode);
     if (!fn) return COSMOS_ATTN_UNSUPPORTED;

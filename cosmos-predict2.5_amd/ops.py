@@ -15,7 +15,8 @@ import torch
 from . import _lib
 
 _DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
-SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)
+SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)        # backward, RMSNorm + RoPE
+FORWARD_HEAD_DIMS = (16, 32, 64, 128, 256)     # forward + JVP and forward only (256 runs a slower kernel of its own)
 REFERENCE_HEAD_DIMS = (16, 32, 64, 128, 256)  # what the reference accepts (…jvp_triton.py:444-445)
 
 
@@ -83,8 +84,8 @@ def fwd_jvp(
     B, H, Lq, d_qk = q.shape
     Lkv, d_v = v.shape[-2], v.shape[-1]
     assert d_qk in REFERENCE_HEAD_DIMS and d_v in REFERENCE_HEAD_DIMS
-    if d_qk not in SUPPORTED_HEAD_DIMS or d_v not in SUPPORTED_HEAD_DIMS:
-        raise NotImplementedError(f"head dims ({d_qk}, {d_v}): the HIP kernels are built for {SUPPORTED_HEAD_DIMS}")
+    if d_qk not in FORWARD_HEAD_DIMS or d_v not in FORWARD_HEAD_DIMS:
+        raise NotImplementedError(f"head dims ({d_qk}, {d_v}): the HIP kernels are built for {FORWARD_HEAD_DIMS}")
     assert (Lq == Lkv) or (not causal), "Causal cross-attention is currently not supported."
     if not q.is_cuda:
         raise RuntimeError("cosmos attention (HIP) needs tensors on a GPU; there is no CPU path")
@@ -174,8 +175,8 @@ def pack_kv(k: torch.Tensor, v: torch.Tensor) -> PackedKV:
     B, H, Lkv, d_qk = k.shape
     d_v = v.shape[-1]
     assert d_qk in REFERENCE_HEAD_DIMS and d_v in REFERENCE_HEAD_DIMS
-    if d_qk not in SUPPORTED_HEAD_DIMS or d_v not in SUPPORTED_HEAD_DIMS:
-        raise NotImplementedError(f"head dims ({d_qk}, {d_v}): the HIP kernels are built for {SUPPORTED_HEAD_DIMS}")
+    if d_qk not in FORWARD_HEAD_DIMS or d_v not in FORWARD_HEAD_DIMS:
+        raise NotImplementedError(f"head dims ({d_qk}, {d_v}): the HIP kernels are built for {FORWARD_HEAD_DIMS}")
     if not k.is_cuda:
         raise RuntimeError("cosmos attention (HIP) needs tensors on a GPU; there is no CPU path")
     if k.dtype not in _DTYPES:

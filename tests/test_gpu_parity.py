@@ -183,6 +183,30 @@ def test_head_dims(pkg, oracle, gpu, dqk, dv, dtype):
     run_case(pkg, oracle, gpu, (1, 2, 150, dqk), (1, 2, 170, dqk), dv=dv, dtype=dtype, seed=dqk + dv, primal_std=0.5, tangent_std=0.5)
 
 
+@pytest.mark.parametrize("dqk,dv", [(256, 256), (256, 64), (128, 256), (16, 256), (256, 16)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tangents", ["full", "q", "none"])
+def test_head_dim_256(pkg, oracle, gpu, dqk, dv, dtype, tangents):
+    """Head dim 256 (flash_attention_jvp_triton.py:444-445 accepts it) runs a kernel of its own: ragged lengths, more than
+    one key tile, every tangent set."""
+    run_case(pkg, oracle, gpu, (1, 2, 150, dqk), (1, 2, 77, dqk), dv=dv, dtype=dtype, tangents=tangents, seed=dqk + dv)
+    run_case(pkg, oracle, gpu, (2, 1, 33, dqk), (2, 1, 300, dqk), dv=dv, dtype=dtype, tangents=tangents, seed=dqk + dv + 1)
+
+
+def test_head_dim_256_masks_and_reference_shapes(pkg, oracle, gpu):
+    run_case(pkg, oracle, gpu, (1, 2, 200, 256), causal=True, seed=1)
+    run_case(pkg, oracle, gpu, (1, 2, 200, 256), causal=True, tangents="none", seed=2)
+    run_case(pkg, oracle, gpu, (2, 2, 100, 256), (2, 2, 90, 256), key_lens=[64, 7], tangents="q", seed=3)
+    run_case(pkg, oracle, gpu, (1, 2, 1024, 256), seed=4, primal_std=0.5, tangent_std=0.5, sm_scale=0.5)   # the reference's test scale
+    # strided [B, L, H, d] views and [B, L, H, d] output memory
+    q, k, v, tq, tk, tv = oracle.make_inputs((1, 2, 130, 256), seed=5)
+    blhd = lambda x: x.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3).to(gpu)
+    o, to, lse = pkg.fwd_jvp(blhd(q), blhd(k), blhd(v), blhd(tq), blhd(tk), blhd(tv), out_layout="blhd")
+    o_ref, to_ref, _ = oracle.closed_form(q, k, v, tq, tk, tv)
+    check(oracle, "o", o, o_ref)
+    check(oracle, "to", to, to_ref)
+
+
 @pytest.mark.parametrize("tangents", ["none", "q", "kv", "v"])
 @pytest.mark.parametrize("dqk,dv", [(128, 128), (64, 32)])
 def test_tangent_sets(pkg, oracle, gpu, tangents, dqk, dv):

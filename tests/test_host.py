@@ -71,7 +71,7 @@ def test_status_codes_for_bad_descriptors(pkg):
         (dict(tk=fake), L.ST_BAD_ARG),                 # tangent on k without q, v
         (dict(tq=fake), L.ST_BAD_ARG),                 # tangents given but no `to`
         (dict(dtype=7), L.ST_UNSUPPORTED),
-        (dict(d_qk=256), L.ST_UNSUPPORTED),
+        (dict(d_qk=512), L.ST_BAD_SHAPE),
         (dict(d_v=48), L.ST_BAD_SHAPE),
         (dict(causal=1), L.ST_BAD_SHAPE),              # causal needs Lq == Lkv
         (dict(q=0x7F0000000008), L.ST_BAD_STRIDE),     # 8-byte aligned base
@@ -435,8 +435,9 @@ def test_python_argument_checks_mirror_reference(pkg):
         pkg.fwd_jvp(q, q, q[:, :, :4])
     with pytest.raises(AssertionError):                     # head dim outside {16,32,64,128,256} (:444-445)
         pkg.fwd_jvp(q[..., :48], q[..., :48], q)
-    with pytest.raises(NotImplementedError):                # 256 is accepted by the reference but not built here
-        pkg.fwd_jvp(torch.zeros(1, 1, 8, 256, dtype=torch.bfloat16), torch.zeros(1, 1, 8, 256, dtype=torch.bfloat16), q[:, :1])
+    with pytest.raises(RuntimeError, match="GPU"):          # 256 is built for the forward paths: the call gets as far as the device check
+        pkg.fwd_jvp(torch.zeros(1, 1, 8, 256, dtype=torch.bfloat16), torch.zeros(1, 1, 8, 256, dtype=torch.bfloat16),
+                    torch.zeros(1, 1, 8, 256, dtype=torch.bfloat16))
     with pytest.raises(AssertionError, match="Causal cross-attention"):   # :446
         pkg.fwd_jvp(q, q[:, :, :4], q[:, :, :4], causal=True)
     with pytest.raises(AssertionError):                     # tangent shape / stride must match the primal (:447-448)
