@@ -531,6 +531,133 @@ attn_bwd_kernel(const BwdParams p) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------- head dim 256
+// At d = 256 the stationary rows of a wavefront are 128 registers and its accumulators up to 256, and a stream tile is
+// 49 / 97 KB: the kernels above do not fit.  This one is built for being right rather than fast (no Cosmos configuration
+// has this head dim): no LDS, no roles, no barriers.  A workgroup is four wavefronts that serve the SAME 32 stationary
+// rows; each computes the whole 32 x 32 tile of scores and dP for itself (A fragments read straight from the re-tiled
+// stream in memory), forms U = P and W = dS, and accumulates its own quarter of the channels (32-channel blocks w and
+// w + 4).  Same arithmetic and rounding points as attn_bwd_kernel; the head dim is a run-time value.
+constexpr int kWideMaxNC = 16;
+constexpr int kWideWaves = 4;
+constexpr int kWideDbPerWave = 2;
+
+template <typename T, int KIND>
+__global__ void __launch_bounds__(64 * kWideWaves) attn_bwd_wide_kernel(const BwdParams p, int d) {
+    typedef typename VecOf<T>::v8 V8;
+    typedef typename VecOf<T>::v4 V4;
+    constexpr bool DKDV = KIND == KIND_DKDV;
+    const int nc = d / 16, ndb = (d + 31) / 32;
+    const int sp_frags = 2 * nc, op_frags = 2 * ndb * (DKDV ? 2 : 1);
+    const int tile_bytes = (sp_frags + op_frags + (DKDV ? 1 : 0)) * kFragBytes;
+
+    const int pair = blockIdx.x;
+    const int blk = pair % p.n_blk, bh = pair / p.n_blk, b = bh / p.H, h = bh % p.H;   // n_blk: blocks of 32 stationary rows
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 31, hh = lane >> 5;
+    const int row0 = blk * kRows, row = row0 + j;
+    const bool causal = p.causal != 0;
+
+    int t_lo = 0, t_hi = p.n_tiles;
+    if (causal) {
+        if (DKDV) t_lo = row0 / kRows;
+        else { const int lim = (row0 + kRows + kRows - 1) / kRows; t_hi = t_hi < lim ? t_hi : lim; }
+    }
+    V8 b1[kWideMaxNC], b2[kWideMaxNC];   // stationary B operands: (q, dO) rows or (k, v) rows
+    float l2 = INFINITY, dd = 0.f;       // dQ kernel: LSE log2(e) and D of this lane's query (rows past the end: P = 0)
+    {
+        const bool live = row < p.L_stat;
+        const T* p1 = reinterpret_cast<const T*>(p.st1) + (int64_t)b * p.s1_sb + (int64_t)h * p.s1_sh + (int64_t)(live ? row : 0) * p.s1_sl + 8 * hh;
+        const T* p2 = reinterpret_cast<const T*>(p.st2) + (int64_t)b * p.s2_sb + (int64_t)h * p.s2_sh + (int64_t)(live ? row : 0) * p.s2_sl + 8 * hh;
+        const V8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int c = 0; c < kWideMaxNC; ++c) {
+            b1[c] = z; b2[c] = z;
+            if (c < nc && live) { b1[c] = *reinterpret_cast<const V8*>(p1 + 16 * c); b2[c] = *reinterpret_cast<const V8*>(p2 + 16 * c); }
+        }
+        if (!DKDV && live) { const float2 st = p.stats[(int64_t)bh * p.L_stat + row]; l2 = st.x; dd = st.y; }
+    }
+    f32x16 acc1[kWideDbPerWave], acc2[kWideDbPerWave];   // dQ^T | dV^T, dK^T
+#pragma unroll
+    for (int i = 0; i < kWideDbPerWave; ++i) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { acc1[i][e] = 0.f; acc2[i][e] = 0.f; }
+    }
+    const char* const head = p.stream + (size_t)bh * p.n_tiles * tile_bytes;
+    auto frag = [&](const char* tile, int f) { return *reinterpret_cast<const V8*>(tile + (size_t)f * kFragBytes + lane * 16); };
+
+    for (int t = t_lo; t < t_hi; ++t) {
+        const char* const tile = head + (size_t)t * tile_bytes;
+        f32x16 sc, dp;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { sc[e] = 0.f; dp[e] = 0.f; }
+#pragma unroll
+        for (int c = 0; c < kWideMaxNC; ++c) {
+            if (c < nc) {
+                sc = mfma32(frag(tile, c), b1[c], sc);
+                dp = mfma32(frag(tile, nc + c), b2[c], dp);
+            }
+        }
+        float l2v[16], ddv[16];
+        if (DKDV) {   // statistics of the 32 streamed queries: LSE log2(e) at float index 16 hh + e, D at 32 + 16 hh + e
+            const float* st = reinterpret_cast<const float*>(tile + (size_t)(sp_frags + op_frags) * kFragBytes);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) { l2v[e] = st[16 * hh + e]; ddv[e] = st[32 + 16 * hh + e]; }
+        }
+        V8 uf[2], wf[2];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int srow = t * kRows + 8 * (e >> 2) + 4 * hh + (e & 3);   // streamed row of element e
+            const bool ok = DKDV ? (!causal || row <= srow) : (srow < p.L_stream && (!causal || srow <= row));   // key <= query
+            const float se = ok ? sc[e] : -INFINITY;
+            const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(se, p.scale_log2, -(DKDV ? l2v[e] : l2)));
+            const float we = pe * (dp[e] - (DKDV ? ddv[e] : dd));
+            uf[e >> 3][e & 7] = (T)pe;
+            wf[e >> 3][e & 7] = (T)we;
+        }
+#pragma unroll
+        for (int i = 0; i < kWideDbPerWave; ++i) {
+            const int db = wave + kWideWaves * i;
+            if (db < ndb) {
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    if (DKDV) {
+                        acc1[i] = mfma32(frag(tile, sp_frags + 2 * db + c), uf[c], acc1[i]);               // dV^T += dO^T U
+                        acc2[i] = mfma32(frag(tile, sp_frags + 2 * ndb + 2 * db + c), wf[c], acc2[i]);     // dK^T += Q^T W
+                    } else {
+                        acc1[i] = mfma32(frag(tile, sp_frags + 2 * db + c), wf[c], acc1[i]);               // dQ^T += K^T W
+                    }
+                }
+            }
+        }
+    }
+    // dQ = s dQ^T   |   dV = dV^T, dK = s dK^T
+    if (row < p.L_stat) {
+        T* o1 = reinterpret_cast<T*>(p.out1) + (int64_t)b * p.o1_sb + (int64_t)h * p.o1_sh + (int64_t)row * p.o1_sl;
+        T* o2 = DKDV ? reinterpret_cast<T*>(p.out2) + (int64_t)b * p.o2_sb + (int64_t)h * p.o2_sh + (int64_t)row * p.o2_sl : o1;
+        const float s1 = DKDV ? 1.0f : p.sm_scale;
+#pragma unroll
+        for (int i = 0; i < kWideDbPerWave; ++i) {
+            const int db = wave + kWideWaves * i;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int ch = 32 * db + 8 * g + 4 * hh;
+                if (db < ndb && ch < d) {
+                    V4 v1, v2;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        v1[r] = (T)(acc1[i][4 * g + r] * s1);
+                        v2[r] = (T)(acc2[i][4 * g + r] * p.sm_scale);
+                    }
+                    *reinterpret_cast<V4*>(o1 + ch) = v1;
+                    if (DKDV) *reinterpret_cast<V4*>(o2 + ch) = v2;
+                }
+            }
+        }
+    }
+}
+
 // Add the partial sums of the ranges of one stationary row (fixed order), scale, round, store.
 // One thread per (row, 4 channels).
 template <typename T, bool DKDV>
@@ -599,6 +726,12 @@ struct BwdGeom {
         stats_bytes = ((bh * d->Lq * sizeof(float2)) + 1023) / 1024 * 1024;
         q_img_bytes = bh * n_q_tiles * q_tile_bytes;
         k_img_bytes = bh * n_k_tiles * k_tile_bytes;
+        if (d->d == 256) {   // attn_bwd_wide_kernel: blocks of 32 stationary rows, never cut
+            dkdv = Plan{(d->Lkv + kRows - 1) / kRows, (d->Lkv + kRows - 1) / kRows * (int)bh, (d->Lkv + kRows - 1) / kRows * (int)bh, 0, 1};
+            dq = Plan{(d->Lq + kRows - 1) / kRows, (d->Lq + kRows - 1) / kRows * (int)bh, (d->Lq + kRows - 1) / kRows * (int)bh, 0, 1};
+            part_bytes = 0;
+            return;
+        }
         dkdv = plan((d->Lkv + kBlock - 1) / kBlock, (int)bh, n_q_tiles, d->causal != 0);
         dq = plan((d->Lq + kBlock - 1) / kBlock, (int)bh, n_k_tiles, d->causal != 0);
         const size_t p1 = (size_t)dkdv.n_rem * dkdv.splits * kBlock * 2 * d->d * sizeof(float);
@@ -627,8 +760,7 @@ int validate_bwd(const cosmos_attn_bwd_desc* d) {
     if (d->B <= 0 || d->H <= 0 || d->Lq <= 0 || d->Lkv <= 0) return COSMOS_ATTN_BAD_ARG;
     if (!d->q || !d->k || !d->v || !d->o || !d->dout || !d->lse || !d->dq || !d->dk || !d->dv) return COSMOS_ATTN_BAD_ARG;
     if (d->dtype != COSMOS_ATTN_BF16 && d->dtype != COSMOS_ATTN_FP16) return COSMOS_ATTN_UNSUPPORTED;
-    if (d->d == 256) return COSMOS_ATTN_UNSUPPORTED;
-    if (!head_dim_ok(d->d)) return COSMOS_ATTN_BAD_SHAPE;
+    if (!head_dim_ok(d->d) && d->d != 256) return COSMOS_ATTN_BAD_SHAPE;
     if (d->causal && d->Lq != d->Lkv) return COSMOS_ATTN_BAD_SHAPE;
     const void* ptrs[] = {d->q, d->k, d->v, d->o, d->dout, d->dq, d->dk, d->dv};
     for (const void* ptr : ptrs) if (!aligned16(ptr)) return COSMOS_ATTN_BAD_STRIDE;
@@ -660,9 +792,10 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
     hipStream_t stream = (hipStream_t)stream_;
     const BwdGeom g(d);
     const bool bf16 = d->dtype == COSMOS_ATTN_BF16;
+    const bool wide = d->d == 256;
     bwd_kernel_t k_dkdv = bf16 ? pick_bwd<__bf16, KIND_DKDV>(d->d) : pick_bwd<_Float16, KIND_DKDV>(d->d);
     bwd_kernel_t k_dq = bf16 ? pick_bwd<__bf16, KIND_DQ>(d->d) : pick_bwd<_Float16, KIND_DQ>(d->d);
-    if (!k_dkdv || !k_dq) return COSMOS_ATTN_UNSUPPORTED;
+    if (!wide && (!k_dkdv || !k_dq)) return COSMOS_ATTN_UNSUPPORTED;
     char* ws = (char*)workspace;
     float2* stats = (float2*)ws;
     char* q_img = ws + g.stats_bytes;
@@ -671,6 +804,12 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
     const int BH = d->B * d->H;
     auto launch = [&](bwd_kernel_t fn, size_t lds, const BwdGeom::Plan& pl, BwdParams& bp, bool is_dkdv) {
         bp.n_blk = pl.n_blk; bp.n_full = pl.n_full; bp.n_rem = pl.n_rem; bp.splits = pl.splits; bp.part = part;
+        if (wide) {
+            auto wfn = is_dkdv ? (bf16 ? attn_bwd_wide_kernel<__bf16, KIND_DKDV> : attn_bwd_wide_kernel<_Float16, KIND_DKDV>)
+                               : (bf16 ? attn_bwd_wide_kernel<__bf16, KIND_DQ> : attn_bwd_wide_kernel<_Float16, KIND_DQ>);
+            hipLaunchKernelGGL(wfn, dim3((unsigned)pl.n_pairs), dim3(64 * kWideWaves), 0, stream, bp, (int)d->d);
+            return true;
+        }
         if (!allow_lds((const void*)fn, lds)) return false;
         hipLaunchKernelGGL(fn, dim3((unsigned)(pl.n_full + pl.n_rem * pl.splits)), dim3(kBwdThreads), lds, stream, bp);
         if (pl.splits > 1) {

@@ -15,8 +15,8 @@ import torch
 from . import _lib
 
 _DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
-SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)        # backward, RMSNorm + RoPE
-FORWARD_HEAD_DIMS = (16, 32, 64, 128, 256)     # forward + JVP and forward only (256 runs a slower kernel of its own)
+SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)        # RMSNorm + RoPE
+FORWARD_HEAD_DIMS = (16, 32, 64, 128, 256)     # attention: forward + JVP, forward only, backward (256 runs slower kernels of its own)
 REFERENCE_HEAD_DIMS = (16, 32, 64, 128, 256)  # what the reference accepts (…jvp_triton.py:444-445)
 
 
@@ -263,8 +263,8 @@ def bwd(
     assert k.shape == (B, H, Lkv, d) and v.shape == (B, H, Lkv, d)
     assert o.shape == q.shape and dout.shape == q.shape and lse.shape == (B, H, Lq)
     assert d in REFERENCE_HEAD_DIMS
-    if d not in SUPPORTED_HEAD_DIMS:
-        raise NotImplementedError(f"head dim {d}: the HIP kernels are built for {SUPPORTED_HEAD_DIMS}")
+    if d not in FORWARD_HEAD_DIMS:
+        raise NotImplementedError(f"head dim {d}: the HIP kernels are built for {FORWARD_HEAD_DIMS}")
     assert (Lq == Lkv) or (not causal), "Causal cross-attention is currently not supported."
     if not q.is_cuda:
         raise RuntimeError("cosmos attention (HIP) needs tensors on a GPU; there is no CPU path")

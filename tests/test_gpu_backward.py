@@ -61,6 +61,20 @@ def test_bwd_head_dims(pkg, oracle, gpu, d, dtype):
     run_bwd(pkg, oracle, gpu, (2, 2, 200, d), (2, 2, 333, d), seed=d, dtype=dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_bwd_head_dim_256(pkg, oracle, gpu, dtype):
+    """Head dim 256 runs kernels of its own: ragged lengths, several stream tiles, causal, through autograd."""
+    run_bwd(pkg, oracle, gpu, (1, 2, 150, 256), (1, 2, 77, 256), dtype=dtype, seed=1)
+    run_bwd(pkg, oracle, gpu, (2, 1, 33, 256), (2, 1, 300, 256), dtype=dtype, seed=2)
+    run_bwd(pkg, oracle, gpu, (1, 2, 200, 256), causal=True, dtype=dtype, seed=3)
+    run_bwd(pkg, oracle, gpu, (1, 2, 1024, 256), dtype=dtype, seed=4, primal_std=0.5, sm_scale=0.5)
+    q, k, v, tq, tk, tv = (x.to(gpu) for x in oracle.make_inputs((1, 2, 100, 256), seed=5, dtype=dtype))
+    qg = q.clone().requires_grad_(True)
+    o, to = pkg.attention_jvp(qg, k, v, tq, tk, tv)
+    o.float().sum().backward()
+    assert qg.grad is not None and torch.isfinite(qg.grad.float()).all()
+
+
 @pytest.mark.parametrize("L", [1, 33, 128, 200, 515])
 def test_bwd_causal(pkg, oracle, gpu, L):
     run_bwd(pkg, oracle, gpu, (1, 2, L, 64), causal=True, seed=L)

@@ -120,7 +120,7 @@ def test_bwd_desc_layout_and_status_codes(pkg):
         (dict(lse=None), L.ST_BAD_ARG),
         (dict(dk=None), L.ST_BAD_ARG),
         (dict(dtype=5), L.ST_UNSUPPORTED),
-        (dict(d=256), L.ST_UNSUPPORTED),
+        (dict(d=512), L.ST_BAD_SHAPE),
         (dict(d=48), L.ST_BAD_SHAPE),
         (dict(causal=1), L.ST_BAD_SHAPE),
         (dict(dout=0x7F0000000004), L.ST_BAD_STRIDE),
