@@ -71,7 +71,7 @@ __device__ __forceinline__ void round4(float* f) {
     unpack4<BF16>(r, f);
 }
 
-// Sum over the TPR (2, 4, 8 or 16) adjacent lanes of a thread group, result in every lane, by data-parallel-primitive
+// Sum over the TPR (2, 4, 8, 16 or 32) adjacent lanes of a thread group, result in every lane, by data-parallel-primitive
 // lane permutations (no LDS traffic): swap within pairs, swap pairs within quads, mirror within 8, mirror within 16.
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
@@ -84,6 +84,7 @@ __device__ __forceinline__ float group_sum(float v) {
     if (TPR >= 4) v = dpp_add<0x4E>(v);    // quad_perm [2, 3, 0, 1]
     if (TPR >= 8) v = dpp_add<0x141>(v);   // row_half_mirror
     if (TPR >= 16) v = dpp_add<0x140>(v);  // row_mirror
+    if (TPR >= 32) v += __shfl_xor(v, 16);  // the other row of 16 lanes (head dim 256 only)
     return v;
 }
 
@@ -92,7 +93,7 @@ __device__ __forceinline__ float group_sum(float v) {
 // sets the time), so the work per element is kept minimal: the element type is a template parameter, the sines and
 // cosines are shared by all heads of a position, and the rotation needs no exchange between lanes.
 //
-// TPR = D / 8 threads per row (2, 4, 8 or 16: a power of two that divides the wavefront).  Thread `part` holds both
+// TPR = D / 8 threads per row (2, 4, 8, 16 or 32: a power of two that divides the wavefront).  Thread `part` holds both
 // members of four rotation pairs: elements [4 part, 4 part + 4) and [D/2 + 4 part, D/2 + 4 part + 4); the row statistics
 // are summed over the TPR lanes by lane permutations.  A thread group serves `heads_per_unit` consecutive heads of one
 // (batch, position), kHeadsPerStep at a time; the loads of a step are issued before their first use.
@@ -216,6 +217,7 @@ norm_rope_kernel_t pick(int d) {
         case 32: return norm_rope_kernel<4, TANGENT, BF16>;
         case 64: return norm_rope_kernel<8, TANGENT, BF16>;
         case 128: return norm_rope_kernel<16, TANGENT, BF16>;
+        case 256: return norm_rope_kernel<32, TANGENT, BF16>;
         default: return nullptr;
     }
 }
@@ -367,6 +369,7 @@ norm_rope_bwd_kernel_t pick_bwd(int d) {
         case 32: return norm_rope_bwd_kernel<4, BF16>;
         case 64: return norm_rope_bwd_kernel<8, BF16>;
         case 128: return norm_rope_bwd_kernel<16, BF16>;
+        case 256: return norm_rope_bwd_kernel<32, BF16>;
         default: return nullptr;
     }
 }
@@ -401,8 +404,7 @@ COSMOS_ATTN_API int cosmos_norm_rope(const cosmos_norm_rope_desc* d, void* strea
     if (!d->x || !d->y || (d->tx != nullptr) != (d->ty != nullptr)) return COSMOS_ATTN_BAD_ARG;
     if (!(d->eps >= 0.f)) return COSMOS_ATTN_BAD_ARG;
     if (d->dtype != COSMOS_ATTN_BF16 && d->dtype != COSMOS_ATTN_FP16) return COSMOS_ATTN_UNSUPPORTED;
-    if (d->D == 256) return COSMOS_ATTN_UNSUPPORTED;
-    if (d->D != 16 && d->D != 32 && d->D != 64 && d->D != 128) return COSMOS_ATTN_BAD_SHAPE;
+    if (d->D != 16 && d->D != 32 && d->D != 64 && d->D != 128 && d->D != 256) return COSMOS_ATTN_BAD_SHAPE;
     if (!aligned16(d->x) || !aligned16(d->y) || (d->tx && (!aligned16(d->tx) || !aligned16(d->ty)))) return COSMOS_ATTN_BAD_STRIDE;
     if (d->angles && !aligned16(d->angles)) return COSMOS_ATTN_BAD_STRIDE;
     if (!strides_ok(d->x_stride) || !strides_ok(d->y_stride)) return COSMOS_ATTN_BAD_STRIDE;
@@ -430,8 +432,7 @@ static int validate_norm_rope_bwd(const cosmos_norm_rope_bwd_desc* d) {
     if (!d->x || !d->dy || !d->dx) return COSMOS_ATTN_BAD_ARG;
     if (!(d->eps >= 0.f)) return COSMOS_ATTN_BAD_ARG;
     if (d->dtype != COSMOS_ATTN_BF16 && d->dtype != COSMOS_ATTN_FP16) return COSMOS_ATTN_UNSUPPORTED;
-    if (d->D == 256) return COSMOS_ATTN_UNSUPPORTED;
-    if (d->D != 16 && d->D != 32 && d->D != 64 && d->D != 128) return COSMOS_ATTN_BAD_SHAPE;
+    if (d->D != 16 && d->D != 32 && d->D != 64 && d->D != 128 && d->D != 256) return COSMOS_ATTN_BAD_SHAPE;
     if (!aligned16(d->x) || !aligned16(d->dy) || !aligned16(d->dx)) return COSMOS_ATTN_BAD_STRIDE;
     if (d->angles && !aligned16(d->angles)) return COSMOS_ATTN_BAD_STRIDE;
     if (!strides_ok(d->x_stride) || !strides_ok(d->dy_stride) || !strides_ok(d->dx_stride)) return COSMOS_ATTN_BAD_STRIDE;

@@ -15,8 +15,8 @@ import torch
 from . import _lib
 
 _DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
-SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)        # RMSNorm + RoPE
-FORWARD_HEAD_DIMS = (16, 32, 64, 128, 256)     # attention: forward + JVP, forward only, backward (256 runs slower kernels of its own)
+SUPPORTED_HEAD_DIMS = (16, 32, 64, 128, 256)   # (attention at 256 runs slower kernels of its own)
+FORWARD_HEAD_DIMS = SUPPORTED_HEAD_DIMS
 REFERENCE_HEAD_DIMS = (16, 32, 64, 128, 256)  # what the reference accepts (…jvp_triton.py:444-445)
 
 

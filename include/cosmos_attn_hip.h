@@ -35,7 +35,7 @@ enum cosmos_attn_dtype {
 enum cosmos_attn_status {
     COSMOS_ATTN_OK = 0,
     COSMOS_ATTN_BAD_ARG = 1,        /* null pointer / negative size */
-    COSMOS_ATTN_BAD_SHAPE = 2,      /* head dim not in {16,32,64,128}, causal with Lq != Lkv */
+    COSMOS_ATTN_BAD_SHAPE = 2,      /* head dim not in {16,32,64,128,256}, causal with Lq != Lkv */
     COSMOS_ATTN_BAD_STRIDE = 3,     /* misaligned base or stride (16-byte rows required) */
     COSMOS_ATTN_UNSUPPORTED = 4,    /* dtype / head-dim combination not built */
     COSMOS_ATTN_WORKSPACE_TOO_SMALL = 5,
@@ -60,7 +60,7 @@ typedef struct cosmos_attn_desc {
     int32_t dtype;           /* enum cosmos_attn_dtype */
     int32_t B, H;            /* batch, heads                                   (JVP:489-490) */
     int32_t Lq, Lkv;         /* query / key sequence lengths                   (JVP:491-492) */
-    int32_t d_qk, d_v;       /* head dims, each in {16,32,64,128}              (JVP:444-445, 256 not built) */
+    int32_t d_qk, d_v;       /* head dims, each in {16,32,64,128,256}          (JVP:444-445; 256 runs a slower kernel) */
     int32_t causal;          /* 1: key j visible to query i iff j <= i; needs Lq == Lkv (JVP:446) */
     float sm_scale;          /* softmax scale; caller resolves the default d_qk^-0.5 (JVP:449-450) */
 
@@ -142,7 +142,7 @@ typedef struct cosmos_attn_bwd_desc {
     int32_t dtype;           /* enum cosmos_attn_dtype: element type of q, k, v, o, dout, dq, dk, dv */
     int32_t B, H;
     int32_t Lq, Lkv;
-    int32_t d;               /* head dim of q, k and v, in {16,32,64,128} */
+    int32_t d;               /* head dim of q, k and v, in {16,32,64,128,256} */
     int32_t causal;
     float sm_scale;          /* the forward's softmax scale (`ctx.sm_scale`, JVP:499) */
     int32_t reserved;        /* 0 */
@@ -174,7 +174,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc *desc, void *work
 typedef struct cosmos_norm_rope_desc {
     int32_t abi_version;     /* COSMOS_ATTN_ABI_VERSION */
     int32_t dtype;           /* enum cosmos_attn_dtype: element type of x, tx, y, ty */
-    int32_t B, S, H, D;      /* D in {16,32,64,128} */
+    int32_t B, S, H, D;      /* D in {16,32,64,128,256} */
     float eps;               /* 1e-6 in the DiT */
     int32_t reserved;        /* 0 */
     const void *x, *tx;      /* device; tx may be NULL (then ty must be NULL) */

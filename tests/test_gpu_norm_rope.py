@@ -98,7 +98,7 @@ def test_smallest(pkg, nr_oracle, gpu):
     run_case(pkg, nr_oracle, gpu, 1, 1, 1, 128)
 
 
-@pytest.mark.parametrize("D", [16, 32, 64, 128])
+@pytest.mark.parametrize("D", [16, 32, 64, 128, 256])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_head_dims_and_dtypes(pkg, nr_oracle, gpu, D, dtype):
     run_case(pkg, nr_oracle, gpu, 2, 37, 3, D, dtype=dtype, seed=D)
@@ -243,7 +243,7 @@ def run_bwd_case(pkg, nr_oracle, gpu, B, S, H, D, dtype=torch.bfloat16, rope=Tru
     return dx, dw
 
 
-@pytest.mark.parametrize("D", [16, 32, 64, 128])
+@pytest.mark.parametrize("D", [16, 32, 64, 128, 256])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_bwd_head_dims_and_dtypes(pkg, nr_oracle, gpu, D, dtype):
     run_bwd_case(pkg, nr_oracle, gpu, 2, 37, 3, D, dtype=dtype, seed=D)

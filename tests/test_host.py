@@ -165,7 +165,7 @@ def test_norm_rope_desc_layout_and_status_codes(pkg):
         (dict(tx=0x7F0000200000), L.ST_BAD_ARG),          # a tangent in without a tangent out
         (dict(eps=-1.0), L.ST_BAD_ARG),
         (dict(dtype=5), L.ST_UNSUPPORTED),
-        (dict(D=256), L.ST_UNSUPPORTED),
+        (dict(D=512), L.ST_BAD_SHAPE),
         (dict(D=48), L.ST_BAD_SHAPE),
         (dict(x=0x7F0000000004), L.ST_BAD_STRIDE),
         (dict(angles=0x7F0000300008), L.ST_BAD_STRIDE),
@@ -202,7 +202,7 @@ def test_norm_rope_bwd_desc_layout_and_status_codes(pkg):
         (dict(H=0), L.ST_BAD_ARG),
         (dict(dy=None), L.ST_BAD_ARG),
         (dict(dtype=5), L.ST_UNSUPPORTED),
-        (dict(D=256), L.ST_UNSUPPORTED),
+        (dict(D=512), L.ST_BAD_SHAPE),
         (dict(D=24), L.ST_BAD_SHAPE),
         (dict(dx=0x7F0000200008), L.ST_BAD_STRIDE),
         (dict(dy_stride=(ctypes.c_int64 * 3)(100 * 6 * 66, 6 * 66, 66)), L.ST_BAD_STRIDE),
@@ -223,8 +223,8 @@ def test_norm_rope_argument_checks(pkg):
         pkg.norm_rope(x, weight=torch.ones(32))
     with pytest.raises(AssertionError, match="one angle per"):
         pkg.norm_rope(x, rope_emb=torch.zeros(4, 1, 1, 64))
-    with pytest.raises(NotImplementedError):
-        pkg.norm_rope(torch.zeros(1, 8, 2, 256, dtype=torch.bfloat16))
+    with pytest.raises(AssertionError):                              # head dim outside {16, 32, 64, 128, 256}
+        pkg.norm_rope(torch.zeros(1, 8, 2, 48, dtype=torch.bfloat16))
 
 
 def test_dit_attention_module_mirrors_reference_surface(pkg):
