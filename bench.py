@@ -36,10 +36,11 @@ PEAK_BF16_TFLOPS = 256 * 4096 * 2.4e9 / 1e12
 # with the 1 GiB copy of --copy-calib) whose summary is the named file; the JSON line carries the file name next to the
 # number ("traffic_source").  A workload without a counter run reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "c3": ((2 * 3.889e7 + 710400) * 1024, "profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt"),
+    "c3": ((2 * 3.120e7 + 711620) * 1024, "profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt"),
     "nr": ((2 * 359158.94 + 675840.03) * 1024, "profiles/norm_rope_kernel_bf16_d128_workload_nr.txt"),
-    "c2": ((2 * 1.733e6 + 1.997e5) * 1024, "profiles/attn_fwd_sym_kernel_bf16_d128_workload_c2.txt"),
-    "c3b": ((2 * (1.467e7 + 4.082e7) + 3.523e5 + 7.045e5) * 1024, "profiles/attn_bwd_kernel_bf16_d128_workload_c3b.txt"),
+    "c2": ((2 * 1.717e6 + 1.997e5) * 1024, "profiles/attn_fwd_sym_kernel_bf16_d128_workload_c2.txt"),
+    "c5": ((2 * 306898 + 603720) * 1024, "profiles/attn_qstream_kernel_bf16_d128_workload_c5.txt"),
+    "c3b": ((2 * (1.462e7 + 4.142e7) + 3.523e5 + 7.045e5) * 1024, "profiles/attn_bwd_kernel_bf16_d128_workload_c3b.txt"),
 }
 _NO_TRAFFIC = (None, None)
 
@@ -649,7 +650,8 @@ def bench_attention(args, pkg, lib, dev, name, steps, warmup, full=True):
                     "mfma_frac": flops_value / (run_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
     roofline.update({"frac": roofline["achieved"] / roofline["peak"], "traffic": traffic, "traffic_source": traffic_source,
                      "algorithmic_bytes": alg_bytes,
-                     "kernel": ("attn_fwd_sym_kernel" if tangents == "none" and not padded else "attn_fwd_jvp_kernel") + " (+ attn_combine_kernel)",
+                     "kernel": "attn_qstream_kernel" if name == "c5" else
+                               ("attn_fwd_sym_kernel" if tangents == "none" and not padded else "attn_fwd_jvp_kernel") + " (+ attn_combine_kernel)",
                      "kernel_ms_avg": run_avg, "kernel_ms_min": min(run_ms),
                      "kernel_ms_median": sorted(run_ms)[len(run_ms) // 2], "pack_kv_kernel_ms_avg": pack_avg})
     result = {
