@@ -32,6 +32,12 @@ class _KeptResults(threading.local):
 _kept = _KeptResults()
 
 
+def results_are_kept() -> bool:
+    """Is a recording or a replay of attention results under way on this thread?  (Callers that have another way to the
+    kernels than ``attention()`` must not take it then.)"""
+    return _kept.record is not None or _kept.replay is not None
+
+
 @contextlib.contextmanager
 def record_attention_results(store: list):
     """Every ``attention()`` call inside appends its ``(o [B,H,S,D] view of [B,S,H,D] memory, lse [B,H,S])`` to ``store``."""
@@ -60,9 +66,12 @@ class _AttentionFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, causal, softmax_scale):
-        if _kept.replay:
+        if _kept.replay is not None:
+            if not _kept.replay:
+                raise RuntimeError("more attention calls in the recomputation than were recorded")
             o, lse = _kept.replay.pop(0)
-            assert o.shape == (q.shape[0], q.shape[2], q.shape[1], v.shape[3]), "recorded attention result of another call"
+            if o.shape != (q.shape[0], q.shape[2], q.shape[1], v.shape[3]) or o.dtype != q.dtype:
+                raise RuntimeError("recorded attention result of another call (shape or type differs)")
         else:
             o, _, lse = ops.fwd_jvp(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
                                     causal=causal, sm_scale=softmax_scale, out_layout="blhd", need_lse=True)
@@ -121,7 +130,9 @@ def attention(
         return _AttentionFn.apply(q, k, v, causal, softmax_scale)   # the SDPA path of the reference is differentiable too
 
     # [B, S, H, D] -> heads-first views (no copy); the kernel writes [B, S, H, D] memory directly
-    if _kept.replay:      # a recomputation in which q, k, v happen not to need gradients
+    if _kept.replay is not None:      # a recomputation in which q, k, v happen not to need gradients
+        if not _kept.replay:
+            raise RuntimeError("more attention calls in the recomputation than were recorded")
         return _kept.replay.pop(0)[0].transpose(1, 2)
     recording = _kept.record is not None
     o, _, lse = ops.fwd_jvp(

@@ -26,6 +26,7 @@ import torch
 from torch import nn
 
 from . import ops
+from .attention import results_are_kept
 from .attn_op import HipAttnOp
 
 
@@ -174,7 +175,7 @@ class Attention(nn.Module):
 
     def _context_is_fixed(self, x: torch.Tensor, context) -> bool:
         return (context is not None) and isinstance(context, torch.Tensor) and x.is_cuda and not torch.is_grad_enabled() \
-            and isinstance(self.v_norm, nn.Identity)
+            and isinstance(self.v_norm, nn.Identity) and not results_are_kept()
 
     # ------------------------------------------------------------------ the reference's surface
     def compute_qkv(self, x, context=None, rope_emb=None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
@@ -273,7 +274,7 @@ class I2VCrossAttention(Attention):
 
     def forward(self, x, context=None, rope_emb=None, video_size=None):
         del video_size
-        if x.is_cuda and not torch.is_grad_enabled():
+        if x.is_cuda and not torch.is_grad_enabled() and not results_are_kept():
             text_context, img_context = context
             q, _ = self._norm_rope(self._heads(self.q_proj(x)), self.q_norm, rope_emb)
             result = self.attn_op.forward_packed(q, self._packed_context("text", text_context, self.k_proj, self.k_norm, self.v_proj))

@@ -253,20 +253,28 @@ class _BlockRecompute(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, block, x, emb, ctx_text, ctx_img, rope, lora, extra):
+        # the second run must compute what the first one did: nothing random inside, same autocast setting
+        if block.training and any(isinstance(m, nn.Dropout) and m.p > 0 for m in block.modules()):
+            raise NotImplementedError("block checkpointing with active dropout (the recomputation would draw another mask)")
         kept = []
         context = ctx_text if ctx_img is None else (ctx_text, ctx_img)
         with torch.no_grad(), record_attention_results(kept):
             out = block(x, emb, context, rope, lora, extra)
         ctx.block, ctx.kept = block, kept
-        ctx.inputs = (x, emb, ctx_text, ctx_img, rope, lora, extra)
+        ctx.autocast = (torch.is_autocast_enabled("cuda"), torch.get_autocast_dtype("cuda"))
+        # saved through autograd's own mechanism: an in-place change of an input before the backward pass is an error,
+        # not a silently wrong gradient
+        ctx.save_for_backward(x, emb, ctx_text, ctx_img, rope, lora, extra)
+        ctx.needs = tuple(t is not None and t.requires_grad for t in (x, emb, ctx_text, ctx_img, rope, lora, extra))
         return out
 
     @staticmethod
     def backward(ctx, gout):
-        ins = [None if t is None else t.detach().requires_grad_(t.requires_grad) for t in ctx.inputs]
+        ins = [None if t is None else t.detach().requires_grad_(need) for t, need in zip(ctx.saved_tensors, ctx.needs)]
         x, emb, ctx_text, ctx_img, rope, lora, extra = ins
         context = ctx_text if ctx_img is None else (ctx_text, ctx_img)
-        with torch.enable_grad(), replay_attention_results(ctx.kept):
+        enabled, dtype = ctx.autocast
+        with torch.enable_grad(), torch.autocast("cuda", enabled=enabled, dtype=dtype), replay_attention_results(ctx.kept):
             out = ctx.block(x, emb, context, rope, lora, extra)
         torch.autograd.backward(out, gout)
         return (None,) + tuple(None if t is None else t.grad for t in ins)
