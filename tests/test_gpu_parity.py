@@ -264,7 +264,7 @@ def test_streaming_kernels_key_padding(pkg, oracle, gpu, monkeypatch, lens, tang
     run_case(pkg, oracle, gpu, (2, 3, 1100, 128), (2, 3, Lkv, 128), key_lens=lens, tangents=tangents, seed=sum(lens))
 
 
-@pytest.mark.parametrize("d", [16, 32, 64])
+@pytest.mark.parametrize("d", [16, 32, 64, 128])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("tangents", ["q", "none", "full"])
 def test_streaming_kernels_head_dims(pkg, oracle, gpu, monkeypatch, d, dtype, tangents):
@@ -639,6 +639,23 @@ def test_config2_shape_480p_forward_ragged(pkg, oracle, gpu):
 def test_config4_shape_14b_rms_normed(pkg, oracle, gpu):
     """The 14B configuration differs from the 2B 720p one in H=40 and RMS-normed q/k: 3 heads at L=84480."""
     sampled_rows_check(pkg, oracle, gpu, H=3, Lq=84480, Lkv=84480, tangents="full", rms=True, seed=2, n_blocks=4)
+
+
+@pytest.mark.parametrize("tangents", ["q", "none"])
+def test_config5_all_heads_takes_the_streaming_kernel(pkg, oracle, gpu, tangents):
+    """Configuration 5 with all 16 heads and both batch rows (9376 (query block, head) pairs): the launch the library itself
+    sends to the query-streaming kernel, no override; 16 sampled row blocks over heads and batch rows; and bitwise the same
+    result from the kernel with one workgroup per query block is not expected (another tile order), only the oracle."""
+    import os
+    assert "COSMOS_ATTN_STREAM_CHUNK" not in os.environ
+    g = torch.Generator().manual_seed(1)
+    lens = [int(x) for x in torch.randint(64, 513, (2,), generator=g)]
+    sampled_rows_check(pkg, oracle, gpu, H=16, Lq=37440, Lkv=512, tangents=tangents, rms=False, key_lens=lens, B=2, seed=4, n_blocks=16)
+
+
+def test_network_shaped_cross_attention_takes_the_streaming_kernel(pkg, oracle, gpu):
+    """The cross-attention call inside the 2B DiT at 720p: B=1, H=16, Lq=84480, Lkv=512, no padding mask, tangent on q."""
+    sampled_rows_check(pkg, oracle, gpu, H=16, Lq=84480, Lkv=512, tangents="q", rms=False, B=1, seed=5, n_blocks=8)
 
 
 def test_config5_shape_cross_attention_key_padding(pkg, oracle, gpu):
