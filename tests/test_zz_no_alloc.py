@@ -81,3 +81,30 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit(pkg, oracle, gpu):
     assert "static scratch" in L.status_string(rc)
     D.abi_version = 0
     assert lib.cosmos_attn_fwd_jvp_static(ctypes.byref(D), None) == L.ST_BAD_ARG
+
+
+def test_static_scratch_entry_point_under_graph_capture(pkg, oracle, gpu, monkeypatch):
+    """What the entry point is for: a HIP graph captured around it (no allocation inside the capture: the outputs exist
+    already), replayed with new input contents and eager work in between, matches eager calls bit for bit.  The streaming
+    kernel is forced so that the capture holds the cross-attention path."""
+    monkeypatch.setenv("COSMOS_ATTN_STREAM_CHUNK", "3")
+    L, lib = pkg._lib, pkg._lib.load_library()
+    make = lambda seed: [x.to(gpu) for x in oracle.make_inputs((2, 2, 900, 128), (2, 2, 200, 128), seed=seed)[:4]]
+    q, k, v, tq = make(0)
+    kl = torch.tensor([200, 90], dtype=torch.int32, device=gpu)
+    o, to, lse = torch.empty_like(q), torch.empty_like(q), torch.empty(q.shape[:3], device=gpu)
+    D = _desc(L, q, k, v, tq, None, None, o, to, lse, kl)
+    assert lib.cosmos_attn_fwd_jvp_static(ctypes.byref(D), torch.cuda.current_stream().cuda_stream) == 0   # eager warm-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        assert lib.cosmos_attn_fwd_jvp_static(ctypes.byref(D), torch.cuda.current_stream().cuda_stream) == 0
+    for seed in (1, 2, 3):
+        fresh = make(seed)
+        for dst, src in zip((q, k, v, tq), fresh):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        o_e, to_e, lse_e = pkg.fwd_jvp(*fresh, key_lens=kl)   # eager work between replays (its own workspace)
+        torch.cuda.synchronize()
+        assert torch.equal(o, o_e) and torch.equal(to, to_e) and torch.equal(lse, lse_e), seed
