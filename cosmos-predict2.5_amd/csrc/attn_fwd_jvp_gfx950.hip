@@ -141,7 +141,7 @@ struct AttnParams {
     // `splits` key ranges, one workgroup each, which leave unnormalised partial results for attn_combine_kernel.
     // slot = (pair - n_full) * splits + split; block_m = query rows per workgroup (128, or 384 forward only)
     int n_qt, n_full, n_rem, splits;
-    // attn_qstream_kernel: workgroup id = chunk * BH + (batch * H + head); a chunk is q_chunk consecutive query blocks
+    // attn_qstream_kernel: BH = batch * heads (the kernel deals the (query block, head) pairs out over its workgroups itself)
     int BH, q_chunk;
     float* part_acc;           // [slot][block_m][d_v] accumulators; with tangents [slot][block_m][2][d_v] (O, T)
     float4* part_stat;         // [slot][block_m]: (running max in log2 units, row sum of P, row sum of H, 0)
@@ -610,7 +610,7 @@ attn_fwd_jvp_kernel(const AttnParams p) {
 // Short key sequences (text cross-attention: a few hundred keys against tens of thousands of queries).  With 16 key
 // tiles per query block the kernel above spends more time starting and finishing a workgroup (query load, first fills,
 // normalisation, output stores: none of it overlapped with anything) than sweeping the keys.  Here a workgroup keeps
-// going: it serves `q_chunk` consecutive query blocks of one (batch, head) as ONE stream of steps.  The K/V tiles of the
+// going: it serves a run of consecutive query blocks of one (batch, head) as ONE stream of steps.  The K/V tiles of the
 // head keep circulating through the LDS rings without a gap (the sweep of the next query block starts where the last
 // one ended, modulo the tile count).  Same roles, rings, hand-over and arithmetic as attn_fwd_jvp_kernel; no causal
 // mask, no key-range split.  All three tangent modes (forward only runs here too: at these lengths the fixed costs
@@ -629,6 +629,9 @@ attn_fwd_jvp_kernel(const AttnParams p) {
 // step.  In every mode the score wavefront fetches the next block's Q / dQ rows into the registers of the current ones,
 // d chunk by d chunk, as the block's last score computation lets go of them (no second register set, no copies).
 // For all this a block has at least two steps (a row of at most 32 keys walks a second, fully masked tile).
+constexpr int kNumXCDs = 8;           // MI355X: 8 accelerator dies of 32 compute units, workgroup ids dealt round-robin
+constexpr int kStreamBlockCost = 5;   // what starting and finishing a query block costs, in half steps (measured: about 2.5 steps)
+
 template <int DV, int MODE>
 struct StreamStores {
     static constexpr bool JVP = MODE != MODE_FWD;
@@ -669,17 +672,56 @@ attn_qstream_kernel(const AttnParams p) {
     constexpr int WAIT_FILLS_STORES = ((IN_FLIGHT + N_STORES) & 15) | (((IN_FLIGHT + N_STORES) >> 4) << 14) | 0x0F70;
 
     const int bid = blockIdx.x;
-    const int bh = bid % p.BH, chunk = bid / p.BH, b = bh / p.H, h = bh % p.H;
-    const int qt0 = chunk * p.q_chunk;                                         // first query block of this workgroup
-    const int nq = p.n_qt - qt0 < p.q_chunk ? p.n_qt - qt0 : p.q_chunk;        // query blocks of this workgroup (>= 1)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const bool score_role = wave < 4;
     const int qw = wave & 3;
     const int j = lane & 31, hh = lane >> 5;
 
+    // Which (query block, head) pairs this workgroup serves.  All pairs, in the order (batch, head, query block), form one
+    // line of work; a pair of batch row b weighs 2 n_b + kStreamBlockCost half steps (n_b key tiles per block, plus what
+    // starting and finishing a block costs), and the gridDim.x workgroups cut the line into pieces of equal weight (the
+    // host launches a multiple of the number of compute units: no thin last round, whatever the key lengths of the rows).
+    // A piece may run over the end of a head: the workgroup then serves it as several streams, one after the other.
+    auto tiles_of = [&](int bb) {
+        int len = p.Lkv;
+        if (p.key_lens) { const int kl = __builtin_amdgcn_readfirstlane(p.key_lens[bb]); len = kl < len ? (kl < 0 ? 0 : kl) : len; }
+        const int nt = (len + kBlockN - 1) / kBlockN;
+        return nt < 2 ? 2 : nt;
+    };
+    // (everything below is the same in all lanes; said explicitly, so that it lives in scalar registers)
+    auto uniform64 = [](int64_t v) {
+        const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)((uint64_t)v >> 32));
+        return (int64_t)(((uint64_t)hi << 32) | lo);
+    };
+    const int n_batch = p.BH / p.H;
+    const int64_t per_row = (int64_t)p.H * p.n_qt;          // pairs of one batch row
+    int64_t total_w = 0;
+    for (int bb = 0; bb < n_batch; ++bb) total_w += per_row * (2 * tiles_of(bb) + kStreamBlockCost);
+    // first pair at or after weight position x on the line
+    auto locate = [&](int64_t x) {
+        int64_t cum = 0;
+        for (int bb = 0; bb < n_batch; ++bb) {
+            const int64_t w = 2 * tiles_of(bb) + kStreamBlockCost, span = per_row * w;
+            if (x < cum + span) return bb * per_row + (x - cum + w - 1) / w;
+            cum += span;
+        }
+        return n_batch * per_row;
+    };
+    // Piece number: workgroups are dealt to the 8 XCDs in turn (id mod 8), and each XCD has an L2 of its own, so the pieces
+    // are numbered such that an XCD's workgroups get one contiguous eighth of the line -- a few heads' K/V images per L2
+    // instead of all of them (the grid is a multiple of 8).
+    const int piece = (bid % kNumXCDs) * ((int)gridDim.x / kNumXCDs) + bid / kNumXCDs;
+    const int64_t pair_lo = uniform64(locate(total_w * piece / (int64_t)gridDim.x)), pair_hi = uniform64(locate(total_w * (piece + 1) / (int64_t)gridDim.x));
+
+    for (int64_t pair = pair_lo; pair < pair_hi;) {
+    const int bh = (int)(pair / p.n_qt), b = bh / p.H, h = bh % p.H;
+    const int qt0 = (int)(pair % p.n_qt);                                      // first query block of this stream
+    const int nq = (int)(pair_hi - pair < (int64_t)(p.n_qt - qt0) ? pair_hi - pair : (int64_t)(p.n_qt - qt0));   // its query blocks (>= 1)
+    pair += nq;
+
     int kv_len = p.Lkv;
-    if (p.key_lens) { const int kl = p.key_lens[b]; kv_len = kl < kv_len ? (kl < 0 ? 0 : kl) : kv_len; }
+    if (p.key_lens) { const int kl = __builtin_amdgcn_readfirstlane(p.key_lens[b]); kv_len = kl < kv_len ? (kl < 0 ? 0 : kl) : kv_len; }
     // key tiles per query block: at least two (a finished block drains, and the next block's rows arrive, during the
     // sweep).  Tiles past the last valid key are fully masked (a row of at most 32 keys walks one such tile, a row
     // without a single valid key two); past the end of the packed buffer the fills deliver zeros.
@@ -754,22 +796,55 @@ attn_qstream_kernel(const AttnParams p) {
         int warm_q = 0, warm_tq = 0;
         // A finished block drains during steps 1 .. n-1 of the next one, step n-2 excepted (its stores would sit behind
         // that step's row fetches in the memory queue and be waited for together with them): max(1, n-2) steps.
+        // The stores go out in batches of DB (reads from the region first, then the stores: one wait per batch), a whole
+        // number of batches per step.  Everything this wavefront does sits on the critical path of the step (one instruction
+        // every few cycles, whatever its kind), so a store is kept to a handful of instructions: addresses are a scalar
+        // base per head and tensor plus 32-bit offsets, batch and store numbers are compile-time inside a batch.
+        constexpr int DB = ST::NS < 4 ? ST::NS : 4;
+        static_assert(ST::RPS >= ST::CPR || (DB * ST::RPS) % ST::CPR == 0, "the swizzle key of a batch's stores depends on the position in the batch only");
         const int drain_steps = n > 3 ? n - 2 : 1;
-        const int st_per_step = (ST::NS + drain_steps - 1) / drain_steps;
+        const int st_per_step = ((ST::NS + drain_steps - 1) / drain_steps + DB - 1) / DB * DB;
         // store number i of a query block's results: tensor i / SPT, rows (i % SPT) RPS .. + RPS - 1 of this wavefront's 32;
         // lane l stores chunk l % CPR of row l / CPR of those
         const int rr = lane / ST::CPR, ch = lane % ST::CPR;
         const unsigned x_lane = rr * ST::ROW_BYTES + ((ch ^ (rr & (ST::CPR - 1))) << 4);
         const unsigned o_lane = ((unsigned)rr * (unsigned)p.o_sl + 8u * ch) * 2u;
         const int64_t o_head = ((int64_t)b * p.o_sb + (int64_t)h * p.o_sh) * 2;
+        char* const o_base = reinterpret_cast<char*>(p.o) + o_head;
+        char* const to_base = reinterpret_cast<char*>(JVP ? p.to : p.o) + o_head;
+        const unsigned o_rps = (unsigned)ST::RPS * (unsigned)p.o_sl * 2u;       // bytes from one store's rows to the next one's
+        auto drain_batch = [&](int qt, int i0, auto whole) {
+            // store i0 + k: tensor t, row group g.  A batch lies inside one tensor (t and the first group g0 are scalars, the
+            // rest compile-time) unless a tensor has fewer stores than a batch: then there is one batch, i0 = 0.
+            constexpr bool ONE_T = ST::SPT >= DB;
+            const int t0 = ONE_T ? i0 / ST::SPT : 0, g0 = ONE_T ? i0 % ST::SPT : 0;
+            const char* const src = smem + xp_base + t0 * 32 * ST::ROW_BYTES + g0 * ST::RPS * ST::ROW_BYTES;
+            const int r0 = qt * kBlockM + qw * 32 + g0 * ST::RPS;
+            const unsigned off0 = (unsigned)r0 * (unsigned)p.o_sl * 2u + o_lane;
+            V8 val[DB];
+#pragma unroll
+            for (int k = 0; k < DB; ++k) {
+                const int tk = ONE_T ? 0 : k / ST::SPT, gk = ONE_T ? k : k % ST::SPT;
+                constexpr unsigned none = 0;
+                const unsigned sw = ST::RPS < ST::CPR ? (unsigned)((gk * ST::RPS) & (ST::CPR - 1)) << 4 : none;   // row g RPS + rr has swizzle key (g RPS + rr) mod CPR
+                val[k] = *reinterpret_cast<const V8*>(src + tk * 32 * ST::ROW_BYTES + gk * ST::RPS * ST::ROW_BYTES + (x_lane ^ sw));
+            }
+#pragma unroll
+            for (int k = 0; k < DB; ++k) {
+                const int tk = ONE_T ? t0 : k / ST::SPT, gk = ONE_T ? k : k % ST::SPT;
+                char* const base = tk ? to_base : o_base;
+                const unsigned off = off0 + gk * o_rps;
+                // (a compiler-generated store, not inline assembly: after a store of more than 8 bytes the data registers
+                // must not be overwritten for two cycles, which the compiler only knows to respect for its own stores)
+                if (decltype(whole)::value || r0 + gk * ST::RPS + rr < p.Lq)
+                    __builtin_nontemporal_store(val[k], reinterpret_cast<V8*>(base + off));
+            }
+        };
         auto drain = [&](int qt, int lo, int hi) {
-            for (int i = lo; i < hi; ++i) {
-                const int t = i / ST::SPT, g = i % ST::SPT;
-                const unsigned sw = ST::RPS < ST::CPR ? ((g * ST::RPS) & (ST::CPR - 1)) << 4 : 0;   // row g RPS + rr has swizzle key (g RPS + rr) mod CPR
-                const V8 val = *reinterpret_cast<const V8*>(smem + xp_base + t * 32 * ST::ROW_BYTES + g * ST::RPS * ST::ROW_BYTES + (x_lane ^ sw));
-                const int r0 = qt * kBlockM + qw * 32 + g * ST::RPS;
-                char* const base = reinterpret_cast<char*>(t ? p.to : p.o) + o_head + (int64_t)r0 * p.o_sl * 2;
-                if (r0 + rr < p.Lq) asm volatile("global_store_dwordx4 %0, %1, %2 nt" ::"v"(o_lane), "v"(val), "s"(base) : "memory");
+            if ((qt + 1) * kBlockM <= p.Lq) {       // all rows of the block exist (every block but a head's last)
+                for (int i = lo; i < hi; i += DB) drain_batch(qt, i, std::true_type());
+            } else {
+                for (int i = lo; i < hi; i += DB) drain_batch(qt, i, std::false_type());
             }
         };
 
@@ -954,8 +1029,9 @@ attn_qstream_kernel(const AttnParams p) {
             t_v = wrap_inc(t_v); t_k = wrap_inc(t_k);
         }
         if (TRICKLE) __builtin_amdgcn_s_barrier();   // hands the last block to the score wavefronts
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // drain the (unused) trailing fills before the LDS is released
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // drain the (unused) trailing fills before the LDS is released (or reused by the next stream)
     }
+    }   // streams of this workgroup
 }
 
 #include "attn_wide_gfx950.h"
@@ -1394,23 +1470,27 @@ SplitPlan plan_split(const cosmos_attn_desc* d) {
     s.n_rem = rem; s.n_full = s.n_pairs - rem; s.splits = splits;
     return s;
 }
-// Short key sequences go to attn_qstream_kernel: query blocks per workgroup (0 = use the other kernels).  Enough
-// workgroups for about six rounds on the chip keep the last round's imbalance small (key lengths may differ per batch
-// row), and at least two blocks per workgroup are needed for the streaming to pay.
+// Short key sequences go to attn_qstream_kernel: number of workgroups (0 = use the other kernels).  The kernel cuts the
+// line of (query block, head) pairs into pieces of equal weight itself, so the launch is a small multiple of the number
+// of compute units (every unit gets the same number of equal pieces); it pays from a few blocks per workgroup on.
+// COSMOS_ATTN_STREAM_CHUNK (blocks per workgroup; 1 = off) overrides the choice: tuning and tests.
 constexpr int kStreamMaxTiles = 64;       // up to 2048 keys
-constexpr int kStreamMaxChunk = 16;
-constexpr int kStreamRounds = 6;
-int stream_chunk_of(const cosmos_attn_desc* d) {
+constexpr int kStreamGroupsPerCU = 1;       // one workgroup fills a compute unit (8 wavefronts, 2 per SIMD at 256 registers): a single round
+constexpr int kStreamMinPairs = 1024;     // four blocks per workgroup: from there on the stream is faster than one workgroup per block (measured)
+int stream_groups_of(const cosmos_attn_desc* d) {
     if (d->causal || d->d_qk != d->d_v || n_tiles_of(d) > kStreamMaxTiles) return 0;
     // the kernel addresses q and o inside a head with 32-bit byte offsets
     if ((int64_t)d->Lq * d->q_stride[2] >= ((int64_t)1 << 30) || (int64_t)d->Lq * d->o_stride[2] >= ((int64_t)1 << 30)) return 0;
     const int n_qt = (d->Lq + kBlockM - 1) / kBlockM;
     const int64_t pairs = (int64_t)n_qt * d->B * d->H;
-    int64_t chunk = pairs / (kNumCUs * kStreamRounds);
-    if (const char* e = getenv("COSMOS_ATTN_STREAM_CHUNK")) chunk = atoi(e);
-    if (chunk > kStreamMaxChunk) chunk = kStreamMaxChunk;
-    if (chunk > n_qt) chunk = n_qt;
-    return chunk < 2 ? 0 : (int)chunk;
+    if (const char* e = getenv("COSMOS_ATTN_STREAM_CHUNK")) {
+        const int chunk = atoi(e);
+        if (chunk < 2 || pairs < 2) return 0;
+        const int64_t groups = ((pairs + chunk - 1) / chunk + 7) / 8 * 8;     // a multiple of the number of XCDs
+        return groups > (1 << 30) ? 0 : (int)groups;
+    }
+    if (const char* e = getenv("COSMOS_ATTN_STREAM_GROUPS")) return atoi(e) > 0 ? (atoi(e) + 7) / 8 * 8 : 0;
+    return pairs >= kStreamMinPairs ? kNumCUs * kStreamGroupsPerCU : 0;
 }
 // LDS of attn_qstream_kernel: the layout of attn_fwd_jvp_kernel (AttnCfg::LDS_BYTES) + the per-block statistics slots
 size_t stream_lds_bytes_of(const cosmos_attn_desc* d) {
@@ -1560,14 +1640,13 @@ int run_impl(const cosmos_attn_desc* d, const void* workspace, size_t workspace_
     ap.BH = d->B * d->H; ap.q_chunk = 0;
     ap.n_qt = (d->Lq + kBlockM - 1) / kBlockM; ap.n_full = ap.n_rem = 0; ap.splits = 1;
     ap.part_acc = nullptr; ap.part_stat = nullptr;
-    if (const int chunk = stream_chunk_of(d)) {   // short key sequences: one workgroup streams `chunk` query blocks
+    if (const int groups = stream_groups_of(d)) {   // short key sequences: `groups` workgroups stream the query blocks
         attn_kernel_t sfn = d->dtype == COSMOS_ATTN_BF16 ? pick_stream<__bf16>(d->d_qk, d->d_v, mode)
                                                          : pick_stream<_Float16>(d->d_qk, d->d_v, mode);
         if (sfn) {
             const size_t slds = stream_lds_bytes_of(d);
             if (!allow_lds((const void*)sfn, slds)) return COSMOS_ATTN_LAUNCH_FAILED;
-            ap.q_chunk = chunk;
-            const int64_t sblocks = (int64_t)((ap.n_qt + chunk - 1) / chunk) * ap.BH;
+            const int64_t sblocks = groups;
             hipLaunchKernelGGL(sfn, dim3((unsigned)sblocks), dim3(kAttnThreads), slds, (hipStream_t)stream, ap);
             return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
         }

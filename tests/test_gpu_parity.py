@@ -244,7 +244,7 @@ def test_single_valid_key(pkg, oracle, gpu):
 
 
 # ------------------------------------------------------------------ short key sequences: the query-streaming kernels
-# The library sends a call to the streaming kernels only when it has thousands of (query block, head) pairs; the
+# The library sends a call to the streaming kernels only when it has a thousand (query block, head) pairs or more; the
 # environment variable COSMOS_ATTN_STREAM_CHUNK (query blocks per workgroup, read at every call) forces them on small ones.
 @pytest.mark.parametrize("chunk", [2, 3, 16])
 @pytest.mark.parametrize("tangents", ["q", "none", "full"])
@@ -262,6 +262,17 @@ def test_streaming_kernels_key_padding(pkg, oracle, gpu, monkeypatch, lens, tang
     monkeypatch.setenv("COSMOS_ATTN_STREAM_CHUNK", "4")
     Lkv = max(lens) if max(lens) > 100 else 100
     run_case(pkg, oracle, gpu, (2, 3, 1100, 128), (2, 3, Lkv, 128), key_lens=lens, tangents=tangents, seed=sum(lens))
+
+
+@pytest.mark.parametrize("groups", [8, 40, 256])
+@pytest.mark.parametrize("tangents", ["q", "none", "full"])
+def test_streaming_kernels_pieces_of_equal_weight(pkg, oracle, gpu, monkeypatch, groups, tangents):
+    """COSMOS_ATTN_STREAM_GROUPS sets the number of workgroups directly.  The kernel cuts the line of (query block, head)
+    pairs into that many pieces of equal weight, a pair weighing by its batch row's key length: with rows of 16, 2 and 7
+    key tiles the pieces hold different numbers of blocks, run over head and row boundaries, and with 256 workgroups for
+    174 pairs some are empty."""
+    monkeypatch.setenv("COSMOS_ATTN_STREAM_GROUPS", str(groups))
+    run_case(pkg, oracle, gpu, (3, 2, 900, 128), (3, 2, 512, 128), key_lens=[512, 40, 200], tangents=tangents, seed=groups)
 
 
 @pytest.mark.parametrize("d", [16, 32, 64, 128])
