@@ -628,8 +628,9 @@ attn_fwd_jvp_kernel(const AttnParams p) {
 // With tangents on k and v the output wavefronts store from their accumulators right after a block's last accumulation
 // step.  In every mode the score wavefront fetches the next block's Q / dQ rows into the registers of the current ones,
 // d chunk by d chunk, as the block's last score computation lets go of them (no second register set, no copies).
-// For all this a block has at least two steps (a row of at most 32 keys walks a second, fully masked tile).
+// For all this a block has at least kStreamMinTiles steps (a row of fewer valid tiles walks fully masked ones as well).
 constexpr int kNumXCDs = 8;           // MI355X: 8 accelerator dies of 32 compute units, workgroup ids dealt round-robin
+constexpr int kStreamMinTiles = 3;    // with two steps a block has no step to touch the next rows in, and is slower than with three (measured)
 constexpr int kStreamBlockCost = 5;   // what starting and finishing a query block costs, in half steps (measured: about 2.5 steps)
 
 template <int DV, int MODE>
@@ -687,7 +688,7 @@ attn_qstream_kernel(const AttnParams p) {
         int len = p.Lkv;
         if (p.key_lens) { const int kl = __builtin_amdgcn_readfirstlane(p.key_lens[bb]); len = kl < len ? (kl < 0 ? 0 : kl) : len; }
         const int nt = (len + kBlockN - 1) / kBlockN;
-        return nt < 2 ? 2 : nt;
+        return nt < kStreamMinTiles ? kStreamMinTiles : nt;
     };
     // (everything below is the same in all lanes; said explicitly, so that it lives in scalar registers)
     auto uniform64 = [](int64_t v) {
@@ -722,11 +723,11 @@ attn_qstream_kernel(const AttnParams p) {
 
     int kv_len = p.Lkv;
     if (p.key_lens) { const int kl = __builtin_amdgcn_readfirstlane(p.key_lens[b]); kv_len = kl < kv_len ? (kl < 0 ? 0 : kl) : kv_len; }
-    // key tiles per query block: at least two (a finished block drains, and the next block's rows arrive, during the
-    // sweep).  Tiles past the last valid key are fully masked (a row of at most 32 keys walks one such tile, a row
-    // without a single valid key two); past the end of the packed buffer the fills deliver zeros.
-    int n = kv_len > 0 ? (kv_len + kBlockN - 1) / kBlockN : 1;
-    if (n < 2) n = 2;
+    // key tiles per query block: at least kStreamMinTiles (a finished block drains, and the next block's rows are touched,
+    // fetched and waited for, during the sweep).  Tiles past the last valid key are fully masked; past the end of the
+    // packed buffer the fills deliver zeros.
+    const int n_valid = (kv_len + kBlockN - 1) / kBlockN;
+    const int n = n_valid < kStreamMinTiles ? kStreamMinTiles : n_valid;
     const int n_flat = nq * n;                     // steps of the whole stream: position f = query block f / n, tile f % n
 
     char* const kring = smem + C::KRING_OFF;
@@ -735,7 +736,9 @@ attn_qstream_kernel(const AttnParams p) {
         const_cast<char*>(p.kv) + (size_t)bh * p.n_tiles * TILE_BYTES, 0, p.n_tiles * TILE_BYTES, 0x00020000);
     // position f of the stream reads tile (f + shift) mod n: one shift for all query blocks, so the tiles keep arriving
     // in the same cyclic order across block boundaries and the fills issued ahead of a boundary are the next block's first
-    const int shift = (((bid >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n;
+    // (a sweep with fully masked tiles starts at tile 0: the first tile of a block must have a valid key, or the running max
+    // would still be -inf when the exponentials refer to it)
+    const int shift = n_valid < n ? 0 : (((bid >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n;
     auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane((u + shift) % n); };
     auto wrap_inc = [&](int t) { ++t; return t >= n ? t - n : t; };
     const int k_run = ((qw * C::KP_LOADS) % C::KP_FR) * kFragBytes, v_run = ((qw * C::VP_LOADS) % C::VP_FR) * kFragBytes;
