@@ -360,10 +360,16 @@ struct OutputWave {
 #pragma unroll
         for (int i = 0; i < PD && i < NB; ++i) fetch_group(i, vpart, fa[i], fb[i]);
         if (__any(alpha != 1.0f)) {   // some row's max moved (wavefront-uniform, rare after the first tiles)
+            // v_mul_legacy_f32: 0 * x = 0 for every x, so a factor of zero clears an accumulator whatever it holds (the
+            // query-streaming kernel starts a block that way instead of with a clearing pass of its own); for factors
+            // in (0, 1] it is the ordinary product.
 #pragma unroll
             for (int i = 0; i < NDB; ++i) {
 #pragma unroll
-                for (int e = 0; e < 16; ++e) { acc[i][e] *= alpha; if (JVP) acct[i][e] *= alpha; }
+                for (int e = 0; e < 16; ++e) {
+                    asm("v_mul_legacy_f32 %0, %1, %2" : "=v"(acc[i][e]) : "v"(alpha), "v"(acc[i][e]));
+                    if (JVP) asm("v_mul_legacy_f32 %0, %1, %2" : "=v"(acct[i][e]) : "v"(alpha), "v"(acct[i][e]));
+                }
             }
         }
 #pragma unroll
@@ -861,6 +867,7 @@ attn_qstream_kernel(const AttnParams p) {
         };
         w.scores_plain(sc0, kring);
         fold(sc0, tile_at(0));
+        alpha = 0.0f;                            // a block's first tile: the output wavefront's rescaling pass clears its accumulators
         int f = 0, qi = 0;                       // position in the stream, and its query block
         bool more = nq > 1;                      // is there a block after block qi?
         // Step f = position s_in of block qi's sweep: softmax of the tile at position f (scores in `cur`), scores of position
@@ -914,6 +921,7 @@ attn_qstream_kernel(const AttnParams p) {
                 w.m_run = -INFINITY; w.l_run = 0.f; w.r_run = 0.f;
             }
             if (f + 1 < n_flat) fold(nxt, t_v);
+            if (KIND == 2) alpha = 0.0f;         // the next block's first tile: see above
             t_v = wrap_inc(t_v);   // tile at position f + 2
             ++f;
         };
@@ -1025,8 +1033,7 @@ attn_qstream_kernel(const AttnParams p) {
                         }
                         stored = row0 + 32 <= p.Lq;     // all rows live: every store instruction had a live lane
                     }
-                    zero_acc();
-                    s_in = 0; ++qi;
+                    s_in = 0; ++qi;                    // (the next block's first tile arrives with a factor of zero)
                 }
             }
             t_v = wrap_inc(t_v); t_k = wrap_inc(t_k);
