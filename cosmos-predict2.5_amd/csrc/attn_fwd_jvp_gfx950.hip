@@ -628,15 +628,19 @@ attn_fwd_jvp_kernel(const AttnParams p) {
 // stores then cost their full drain time on top of the sweep).  So, except with tangents on k and v (no LDS left):
 //   * an output wavefront normalises a finished block into a private LDS region (whole rows, 16-byte chunks XOR-swizzled
 //     by row so that neither side has bank conflicts) and goes on accumulating the next block;
-//   * the score wavefront of the pair drains that region to memory a few 1 KB stores per step during the next block's
-//     sweep (16-byte stores covering whole rows).  Its vector-memory counter is not the one that tracks the fills, so
-//     nobody ever waits for a store to retire;
+//   * the score wavefront of the pair drains that region to memory a few 1 KB stores per step during the first steps of
+//     the next block's sweep (16-byte stores covering whole rows).  Its vector-memory counter is not the one that tracks
+//     the fills, so nobody ever waits for a store to retire;
+//   * once the region is empty again, the output wavefront copies the next block's Q / dQ rows into it (direct-to-LDS
+//     loads covering whole rows, one step before the block's end), and the score wavefront reads its fragments from there
+//     at the start of the block's last step, the first to need them.  A block's steps: results of the last block written
+//     to the region / drained / next rows copied / next rows read.
 // With tangents on k and v the output wavefronts store from their accumulators right after a block's last accumulation
-// step.  In every mode the score wavefront fetches the next block's Q / dQ rows into the registers of the current ones,
+// step, and the score wavefront fetches the next block's Q / dQ rows from memory into the registers of the current ones,
 // d chunk by d chunk, as the block's last score computation lets go of them (no second register set, no copies).
 // For all this a block has at least kStreamMinTiles steps (a row of fewer valid tiles walks fully masked ones as well).
 constexpr int kNumXCDs = 8;           // MI355X: 8 accelerator dies of 32 compute units, workgroup ids dealt round-robin
-constexpr int kStreamMinTiles = 3;    // with two steps a block has no step to touch the next rows in, and is slower than with three (measured)
+constexpr int kStreamMinTiles = 4;
 constexpr int kStreamBlockCost = 5;   // what starting and finishing a query block costs, in half steps (measured: about 2.5 steps)
 
 template <int DV, int MODE>
@@ -797,21 +801,26 @@ attn_qstream_kernel(const AttnParams p) {
         w.m_run = -INFINITY;
         w.l_run = 0.f;
         w.r_run = 0.f;
-        // The next block's rows replace the current ones in place: step n-2 of a block computes the block's last scores,
-        // and right after the MFMAs of d chunk c it fetches chunk c of the next block into the same registers; step n-1
-        // (the next block's first scores) then waits chunk by chunk.  That leaves a load one step to arrive, enough from
-        // the L2 but not from memory: step 0 of the block touches every 128-byte line of those rows (4 bytes per lane).
+        // The next block's rows replace the current ones in place.  With tangents on k and v: step n-2 of a block computes
+        // the block's last scores, and right after the MFMAs of d chunk c it fetches chunk c of the next block into the
+        // same registers; step n-1 (the next block's first scores) then waits chunk by chunk.  That leaves a load one step
+        // to arrive, enough from the L2 but not from memory: step 0 of the block touches every 128-byte line of those rows
+        // (4 bytes per lane).  Such a fetch is 16-byte pieces of 32 different rows per instruction, 32 cache lines each:
+        // 2000 cycles per block during which the fills queue up behind it.  In the other modes the rows therefore come
+        // through the LDS region of the pair, which is free once the last block's results have left it: the output
+        // wavefront copies them there during step n-2 with direct-to-LDS loads that cover whole lines (4 rows of 256 bytes
+        // per instruction at d = 128), XOR-swizzled like the results, and this wavefront reads them at the top of step n-1.
+        // The touches stay (the copy then hits the L2).
         constexpr int Q_LINES = (2 * DQK + 127) / 128;   // lines per row (at most 2: lane half hh takes line hh)
         int warm_q = 0, warm_tq = 0;
-        // A finished block drains during steps 1 .. n-1 of the next one, step n-2 excepted (its stores would sit behind
-        // that step's row fetches in the memory queue and be waited for together with them): max(1, n-2) steps.
+        // A finished block drains during steps 1 .. n-3 of the next one (then the region takes the next block's rows).
         // The stores go out in batches of DB (reads from the region first, then the stores: one wait per batch), a whole
         // number of batches per step.  Everything this wavefront does sits on the critical path of the step (one instruction
         // every few cycles, whatever its kind), so a store is kept to a handful of instructions: addresses are a scalar
         // base per head and tensor plus 32-bit offsets, batch and store numbers are compile-time inside a batch.
         constexpr int DB = ST::NS < 4 ? ST::NS : 4;
         static_assert(ST::RPS >= ST::CPR || (DB * ST::RPS) % ST::CPR == 0, "the swizzle key of a batch's stores depends on the position in the batch only");
-        const int drain_steps = n > 3 ? n - 2 : 1;
+        const int drain_steps = n - 3;
         const int st_per_step = ((ST::NS + drain_steps - 1) / drain_steps + DB - 1) / DB * DB;
         // store number i of a query block's results: tensor i / SPT, rows (i % SPT) RPS .. + RPS - 1 of this wavefront's 32;
         // lane l stores chunk l % CPR of row l / CPR of those
@@ -890,7 +899,18 @@ attn_qstream_kernel(const AttnParams p) {
                 warm_q = *reinterpret_cast<const int*>(q_head + off);
                 if (JVP) warm_tq = *reinterpret_cast<const int*>(tq_head + off);
             }
-            if (KIND == 1 && more) {
+            if (KIND == 2 && TRICKLE && more) {
+                // the next block's rows, from the pair's LDS region: 16-byte piece k = 2 c + hh of row j sits at position
+                // k ^ (j mod CPR) of the row
+                const char* const src = smem + xp_base + j * ST::ROW_BYTES;
+#pragma unroll
+                for (int c = 0; c < NC; ++c) {
+                    const unsigned pos = (unsigned)((2 * c + hh) ^ (j & (ST::CPR - 1))) << 4;
+                    w.qf[c] = *reinterpret_cast<const V8*>(src + pos);
+                    if (JVP) w.tqf[c] = *reinterpret_cast<const V8*>(src + 32 * ST::ROW_BYTES + pos);
+                }
+            }
+            if (KIND == 1 && !TRICKLE && more) {
                 const unsigned off = q_off(qt0 + qi + 1);
                 w.step(cur, nxt, kpart, ph_out, alpha_out, alpha, [&](int c) {
                     w.qf[c] = __builtin_nontemporal_load(reinterpret_cast<const V8*>(q_head + off + 32 * c));
@@ -900,8 +920,8 @@ attn_qstream_kernel(const AttnParams p) {
                 w.step(cur, nxt, kpart, ph_out, alpha_out, alpha);
             }
             if (KIND == 2) asm volatile("" ::"v"(warm_q), "v"(warm_tq));   // the touches are done with (keeps their registers theirs until here)
-            if (TRICKLE && KIND != 1 && qi > 0 && s_in > 0) {
-                const int lo = (KIND == 2 ? drain_steps - 1 : s_in - 1) * st_per_step, hi = lo + st_per_step;
+            if (TRICKLE && KIND == 0 && qi > 0 && s_in > 0) {
+                const int lo = (s_in - 1) * st_per_step, hi = lo + st_per_step;
                 drain(qt0 + qi - 1, lo, hi < ST::NS ? hi : ST::NS);
             }
             if (KIND == 2) {
@@ -960,18 +980,53 @@ attn_qstream_kernel(const AttnParams p) {
             }
         };
         zero_acc();
+        // TRICKLE: the next block's Q (and dQ) rows of this pair go to the pair's LDS region during the score wavefront's
+        // step n-2, as direct-to-LDS loads of 1 KB each that cover whole rows (RPS rows per load, SPT loads per tensor):
+        // lane l fills 16-byte position l % CPR of row l / CPR with piece (l % CPR) ^ (row mod CPR) of that row, the
+        // swizzle the results use.  Rows past Lq lie outside the buffer resource and arrive as zeros.
+        const int64_t q_head_off = ((int64_t)b * p.q_sb + (int64_t)h * p.q_sh) * 2;
+        const unsigned q_extent = (unsigned)(p.Lq - 1) * (unsigned)p.q_sl * 2u + 2u * DQK;
+        const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char*>(reinterpret_cast<const char*>(p.q)) + q_head_off, 0, q_extent, 0x00020000);
+        const __amdgpu_buffer_rsrc_t tq_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char*>(reinterpret_cast<const char*>(JVP ? p.tq : p.q)) + q_head_off, 0, q_extent, 0x00020000);
+        const int c_rr = lane / ST::CPR, c_ch = lane % ST::CPR;
+        const unsigned c_row = (unsigned)c_rr * (unsigned)p.q_sl * 2u;
+        const unsigned c_piece = c_ch ^ (c_rr & (ST::CPR - 1));
+        auto copy_rows = [&](int qt) {
+            const unsigned row0 = qt * kBlockM + qw * 32;
+#pragma unroll
+            for (int t = 0; t < ST::NT; ++t) {
+#pragma unroll
+                for (int g = 0; g < ST::SPT; ++g) {
+                    constexpr unsigned none = 0;
+                    const unsigned sw = ST::RPS < ST::CPR ? (unsigned)((g * ST::RPS) & (ST::CPR - 1)) : none;
+                    const int voff = (int)(c_row + ((c_piece ^ sw) << 4));
+                    const int soff = (int)((row0 + g * ST::RPS) * (unsigned)p.q_sl * 2u);
+                    lds_load<0>(t ? tq_rsrc : q_rsrc, smem + xp_base + t * 32 * ST::ROW_BYTES + g * ST::RPS * ST::ROW_BYTES, voff, soff);
+                }
+            }
+        };
+        constexpr int WAIT_COPIED = ((C::KP_LOADS + C::VP_LOADS) & 15) | (((C::KP_LOADS + C::VP_LOADS) >> 4) << 14) | 0x0F70;
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         int qi = 0, s_in = 0;
+        int pos = 0, qb = 0;                     // the score wavefront's position in its block, and that block
         bool stored = false;                     // did the previous step issue output stores? (wavefront-uniform)
+        bool copied = false;                     // did the previous step issue the copy of the next block's rows?
         // Step f: accumulate the tile at position f-1 (P^T, H^T, alpha written by the score wavefront during step f-1);
         // if that was the last tile of its query block, normalise the block, send it off and start the next one from zero.
         for (int f = 0; f <= n_flat; ++f) {
-            if (stored) __builtin_amdgcn_s_waitcnt(WAIT_FILLS_STORES); else __builtin_amdgcn_s_waitcnt(WAIT_FILLS);
-            stored = false;
+            // (after a copy -- issued ahead of that step's fills -- only those fills may still be in flight)
+            if (copied) __builtin_amdgcn_s_waitcnt(WAIT_COPIED);
+            else if (stored) __builtin_amdgcn_s_waitcnt(WAIT_FILLS_STORES);
+            else __builtin_amdgcn_s_waitcnt(WAIT_FILLS);
+            stored = false; copied = false;
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+            if (TRICKLE && pos == n - 2 && qb + 1 < nq) { copy_rows(qt0 + qb + 1); copied = true; }
+            if (++pos == n) { pos = 0; ++qb; }
             issue_group<C>(make_job(t_k, f + 4, t_v, f + 1));
             if (f > 0) {
                 w.step(vring + ((f - 1) % kRingV) * VP_BYTES, smem + ph_base + ((f - 1) & 1) * 4 * C::PH_BYTES,
