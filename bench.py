@@ -39,7 +39,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c3": ((2 * 3.120e7 + 711620) * 1024, "profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt"),
     "nr": ((2 * 359158.94 + 675840.03) * 1024, "profiles/norm_rope_kernel_bf16_d128_workload_nr.txt"),
     "c2": ((2 * 1.717e6 + 1.997e5) * 1024, "profiles/attn_fwd_sym_kernel_bf16_d128_workload_c2.txt"),
-    "c5": ((2 * 305496 + 603781) * 1024, "profiles/attn_qstream_kernel_bf16_d128_workload_c5.txt"),
+    "c5": ((2 * 326847 + 603763) * 1024, "profiles/attn_qstream_kernel_bf16_d128_workload_c5.txt"),
     "c3b": ((2 * (1.462e7 + 4.142e7) + 3.523e5 + 7.045e5) * 1024, "profiles/attn_bwd_kernel_bf16_d128_workload_c3b.txt"),
 }
 _NO_TRAFFIC = (None, None)
