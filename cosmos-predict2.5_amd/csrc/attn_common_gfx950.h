@@ -42,6 +42,15 @@ constexpr float kMaxSlack = 6.0f;
 #ifndef COSMOS_ATTN_PREFETCH_GROUPS
 #define COSMOS_ATTN_PREFETCH_GROUPS 2   // LDS operand fetches run this many MFMA groups ahead of use
 #endif
+// The forward + JVP kernels' two roles have depths of their own.  The output wavefront runs 6 groups ahead (measured at the
+// 2B 720p shape, score / output depth: 2/2 137-138 ms, 4/4 134.6-135, 2/6 133.3, 2/8 133.6, 4/8 134.5): it has the
+// registers for it, and its MFMAs are what fills the gaps the score wavefront leaves in the pipe.
+#ifndef COSMOS_ATTN_PREFETCH_SCORE
+#define COSMOS_ATTN_PREFETCH_SCORE 2
+#endif
+#ifndef COSMOS_ATTN_PREFETCH_OUTPUT
+#define COSMOS_ATTN_PREFETCH_OUTPUT 6
+#endif
 #ifndef COSMOS_ATTN_SWEEP_STAGGER
 #define COSMOS_ATTN_SWEEP_STAGGER 2   // tiles between the sweep starts of workgroups that share an L2
 #endif

@@ -195,7 +195,7 @@ struct ScoreWave {
     typedef typename VecOf<T>::v8 V8;
     static constexpr int NC = C::NC;
     static constexpr bool JVP = C::JVP, FULL = C::FULL;
-    static constexpr int PD = COSMOS_ATTN_PREFETCH_GROUPS;   // LDS operand fetches run this many chunks ahead of use
+    static constexpr int PD = COSMOS_ATTN_PREFETCH_SCORE;    // LDS operand fetches run this many chunks ahead of use
 
     // Scores of one tile as this lane sees them: its query column x 16 of the tile's 32 keys (element e is key
     // 8 (e/4) + 4 (lane/32) + e%4 of the tile) -- the accumulator registers of the score MFMAs themselves.
@@ -336,7 +336,7 @@ struct OutputWave {
     static constexpr int NDB = C::NDB;
     static constexpr bool JVP = C::JVP, FULL = C::FULL;
     static constexpr int NB = 2 * NDB;      // MFMA groups of a step, g = c * NDB + db
-    static constexpr int PD = COSMOS_ATTN_PREFETCH_GROUPS;
+    static constexpr int PD = COSMOS_ATTN_PREFETCH_OUTPUT;
 
     f32x16 acc[NDB], acct[NDB];
     int lane;
