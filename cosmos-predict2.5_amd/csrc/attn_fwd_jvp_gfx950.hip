@@ -881,9 +881,10 @@ attn_qstream_kernel(const AttnParams p) {
         bool more = nq > 1;                      // is there a block after block qi?
         // Step f = position s_in of block qi's sweep: softmax of the tile at position f (scores in `cur`), scores of position
         // f+1 into `nxt`, its statistics.  Three kinds, as separate code: steps 0 .. n-3 of a block; step n-2, which refills
-        // the Q / dQ registers; step n-1, which waits for them chunk by chunk and closes the block.  (Apart, so that the
-        // compiler sees every fetch waited for inside the pair of steps that issues it and puts no waits for it -- which
-        // would wait for the drain stores as well -- into the other steps.)
+        // the Q / dQ registers from memory with tangents on k and v (a plain step otherwise); step n-1, which waits for
+        // them chunk by chunk, or reads them from the LDS region, and closes the block.  (Apart, so that the compiler sees
+        // every fetch waited for inside the pair of steps that issues it and puts no waits for it -- which would wait for
+        // the drain stores as well -- into the other steps.)
         typedef std::integral_constant<int, 0> Plain;
         typedef std::integral_constant<int, 1> Refill;
         typedef std::integral_constant<int, 2> Last;
