@@ -36,9 +36,9 @@ PEAK_BF16_TFLOPS = 256 * 4096 * 2.4e9 / 1e12
 # with the 1 GiB copy of --copy-calib) whose summary is the named file; the JSON line carries the file name next to the
 # number ("traffic_source").  A workload without a counter run reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "c3": ((2 * 3.505e7 + 710583) * 1024, "profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt"),
+    "c3": ((2 * 2.633e7 + 710537) * 1024, "profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt"),
     "nr": ((2 * 359158.94 + 675840.03) * 1024, "profiles/norm_rope_kernel_bf16_d128_workload_nr.txt"),
-    "c2": ((2 * 1.717e6 + 1.997e5) * 1024, "profiles/attn_fwd_sym_kernel_bf16_d128_workload_c2.txt"),
+    "c2": ((2 * 1.770e6 + 1.997e5) * 1024, "profiles/attn_fwd_sym_kernel_bf16_d128_workload_c2.txt"),
     "c5": ((2 * 326847 + 603763) * 1024, "profiles/attn_qstream_kernel_bf16_d128_workload_c5.txt"),
     "c3b": ((2 * (1.462e7 + 4.142e7) + 3.523e5 + 7.045e5) * 1024, "profiles/attn_bwd_kernel_bf16_d128_workload_c3b.txt"),
 }

@@ -52,7 +52,8 @@ constexpr float kMaxSlack = 6.0f;
 #define COSMOS_ATTN_PREFETCH_OUTPUT 6
 #endif
 #ifndef COSMOS_ATTN_SWEEP_STAGGER
-#define COSMOS_ATTN_SWEEP_STAGGER 2   // tiles between the sweep starts of workgroups that share an L2
+#define COSMOS_ATTN_SWEEP_STAGGER 3   // tiles between the sweep starts of workgroups that share an L2 (measured at the 2B 720p
+                                      // shape: same time for 1 .. 4; traffic past the L2 56 / 48 / 36-38 / 26 / 26 / 82 GB at 0 / 1 / 2 / 3 / 4 / 6)
 #endif
 
 #define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)

@@ -641,6 +641,7 @@ attn_fwd_jvp_kernel(const AttnParams p) {
 // For all this a block has at least kStreamMinTiles steps (a row of fewer valid tiles walks fully masked ones as well).
 constexpr int kNumXCDs = 8;           // MI355X: 8 accelerator dies of 32 compute units, workgroup ids dealt round-robin
 constexpr int kStreamMinTiles = 4;
+constexpr int kStreamStagger = 2;     // tiles between the sweep starts of the workgroups of an XCD
 constexpr int kStreamBlockCost = 5;   // what starting and finishing a query block costs, in half steps (measured: about 2.5 steps)
 
 template <int DV, int MODE>
@@ -748,7 +749,7 @@ attn_qstream_kernel(const AttnParams p) {
     // in the same cyclic order across block boundaries and the fills issued ahead of a boundary are the next block's first
     // (a sweep with fully masked tiles starts at tile 0: the first tile of a block must have a valid key, or the running max
     // would still be -inf when the exponentials refer to it)
-    const int shift = n_valid < n ? 0 : (((bid >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n;
+    const int shift = n_valid < n ? 0 : (((bid >> 3) & 31) * kStreamStagger) % n;
     auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane((u + shift) % n); };
     auto wrap_inc = [&](int t) { ++t; return t >= n ? t - n : t; };
     const int k_run = ((qw * C::KP_LOADS) % C::KP_FR) * kFragBytes, v_run = ((qw * C::VP_LOADS) % C::VP_FR) * kFragBytes;
