@@ -188,6 +188,8 @@ struct BwdParams {
 
 extern __shared__ __attribute__((aligned(1024))) char smem[];
 
+constexpr int kBwdSweepStagger = 2;   // tiles between the sweep starts of workgroups that share an L2 (3 as in the forward kernels: dQ kernel 1 % slower, 25 % more traffic)
+
 template <typename T, int D, int KIND>
 struct BwdScoreWave {
     typedef BwdCfg<D, KIND> C;
@@ -383,7 +385,7 @@ attn_bwd_kernel(const BwdParams p) {
     // Sweep order: accumulation is order-free, so workgroups that share an XCD's L2 start a few tiles apart and wrap
     // around (a fixed function of the workgroup id: results stay bitwise reproducible).
     const int n_sweep = n_steps > 0 ? n_steps : 1;
-    const int shift = (((pair >> 3) & 31) * COSMOS_ATTN_SWEEP_STAGGER) % n_sweep;
+    const int shift = (((pair >> 3) & 31) * kBwdSweepStagger) % n_sweep;
     auto tile_at = [&](int u) { return __builtin_amdgcn_readfirstlane(t_lo + (u + shift) % n_sweep); };
     auto wrap_inc = [&](int t) { ++t; return t >= t_lo + n_sweep ? t - n_sweep : t; };
     const int s_run = ((qw * C::SP_LOADS) % C::SP_FR) * kFragBytes, o_run = ((qw * C::OP_LOADS) % C::OP_FR) * kFragBytes;
