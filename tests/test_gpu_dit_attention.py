@@ -175,7 +175,9 @@ def test_fixed_context_is_packed_once_and_reused(pkg, gpu, monkeypatch):
     assert len(calls) == 3                                   # cache off: every call packs
     for x1, x2, x3 in zip(a, b, r):
         assert torch.equal(x1, x2) and torch.equal(x1, x3)
-    assert torch.equal(a[0], a[1])
+    # (forward only and forward + JVP are different kernels, whose workgroups may walk the key tiles in different cyclic
+    # orders: the primal outputs agree to rounding, not bit for bit)
+    torch.testing.assert_close(a[0].float(), a[1].float(), atol=1e-2, rtol=2e-2)
     context.mul_(0.5)                                        # same tensor, new contents
     c = both(m, context)
     assert len(calls) == 4 and not torch.equal(c[0], a[0])
