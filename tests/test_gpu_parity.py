@@ -275,6 +275,25 @@ def test_streaming_kernels_pieces_of_equal_weight(pkg, oracle, gpu, monkeypatch,
     run_case(pkg, oracle, gpu, (3, 2, 900, 128), (3, 2, 512, 128), key_lens=[512, 40, 200], tangents=tangents, seed=groups)
 
 
+@pytest.mark.parametrize("chunk", [0, 1, 2])
+def test_streaming_kernels_random_shapes(pkg, oracle, gpu, monkeypatch, chunk):
+    """36 seeded random cases (12 per chunk) through the streaming kernels: batch, heads, query and key lengths, per-row key
+    lengths, head dim, dtype, tangent set and the number of workgroups drawn at random."""
+    import random
+    rng = random.Random(77 + chunk)
+    for it in range(12):
+        d = rng.choice([16, 32, 64, 128, 128, 128])
+        dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+        tangents = rng.choice(["q", "q", "none", "full"])
+        B, H = rng.choice([1, 2, 3]), rng.choice([1, 2, 3])
+        Lq = rng.choice([1, 37, 128, 129, 300, 640, 777, 1100, 1500])
+        Lkv = rng.choice([17, 32, 33, 64, 65, 96, 100, 128, 160, 200, 257, 384, 512, 700])
+        lens = [rng.randint(2, Lkv) for _ in range(B)] if rng.random() < 0.5 else None
+        monkeypatch.setenv("COSMOS_ATTN_STREAM_GROUPS", str(rng.choice([8, 16, 24, 40, 64, 256])))
+        run_case(pkg, oracle, gpu, (B, H, Lq, d), (B, H, Lkv, d), tangents=tangents, dtype=dtype, key_lens=lens,
+                 seed=9000 + 100 * chunk + it)
+
+
 @pytest.mark.parametrize("d", [16, 32, 64, 128])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("tangents", ["q", "none", "full"])
