@@ -19,7 +19,7 @@ LIB_PATH = os.environ.get("COSMOS_ATTN_LIB") or _BUILT_LIB_PATH
 ABI_VERSION = 2
 DTYPE_BF16, DTYPE_FP16 = 0, 1
 
-ST_OK, ST_BAD_ARG, ST_BAD_SHAPE, ST_BAD_STRIDE, ST_UNSUPPORTED, ST_WORKSPACE, ST_LAUNCH, ST_STATIC_SCRATCH = range(8)
+ST_OK, ST_BAD_ARG, ST_BAD_SHAPE, ST_BAD_STRIDE, ST_UNSUPPORTED, ST_WORKSPACE, ST_LAUNCH, ST_STATIC_SCRATCH, ST_WRONG_DEVICE = range(9)
 
 
 class AttnDesc(ctypes.Structure):
@@ -175,6 +175,7 @@ class GeluDesc(ctypes.Structure):
 EXPORTS = {
     "cosmos_attn_abi_version": (ctypes.c_int, []),
     "cosmos_attn_status_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "cosmos_attn_set_stream_override": (None, [ctypes.c_int, ctypes.c_int]),
     "cosmos_attn_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(AttnDesc)]),
     "cosmos_attn_fwd_jvp": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "cosmos_attn_static_scratch_bytes": (ctypes.c_size_t, []),

@@ -8,14 +8,13 @@ Behaviour kept: cast of q,k,v to ``dtype`` (:110-112), ``q_scale`` (:114-115), `
 unsupported dtypes (:107-108), ``q_lens`` / ``k_lens`` accepted and ignored (:94-95 -- the reference never
 reads them).  The gfx950 kernels are deterministic (no atomics, fixed reduction order), so
 ``deterministic=True`` is honoured instead of raising (:151-154).  fp32 is not built: NotImplementedError.
-``dropout_p`` is accepted and not applied, with one warning: this entry stands where the reference calls Flash
-Attention 3 (:119-127), a call that does not receive ``dropout_p`` either.
+``dropout_p != 0`` raises NotImplementedError: the reference's SDPA branch applies it (:176), the HIP kernels have no
+dropout, and silently returning unregularised attention would be the worse deviation.
 """
 from __future__ import annotations
 
 import contextlib
 import threading
-import warnings
 
 import torch
 
@@ -89,9 +88,6 @@ class _AttentionFn(torch.autograd.Function):
         return t(dq), t(dk), t(dv), None, None
 
 
-_warned_dropout = False
-
-
 def attention(
     q,
     k,
@@ -111,13 +107,9 @@ def attention(
         # kernels compute from 16-bit operands only
         raise NotImplementedError(f"{dtype=} is not supported.")
     if dropout_p != 0.0:
-        # This entry stands where the reference calls Flash Attention 3 (attention.py:119-127), and that call does not
-        # receive dropout_p either: on that branch the argument has no effect.  Same here, said once.
-        global _warned_dropout
-        if not _warned_dropout:
-            _warned_dropout = True
-            warnings.warn("attention(): dropout_p is not applied by the HIP kernels (as on the reference's Flash Attention 3 "
-                          "branch, which does not forward it)", stacklevel=2)
+        # On a ROCm build the reference takes its SDPA branch (get_device_cc() returns 0, attention.py:84-87, :127), which
+        # applies dropout_p (:176).  The HIP kernels have no dropout: refuse loudly rather than train unregularised.
+        raise NotImplementedError(f"attention(): dropout_p={dropout_p} is not supported by the HIP kernels (pass 0.0)")
     del q_lens, k_lens, deterministic
 
     q = q.to(dtype)

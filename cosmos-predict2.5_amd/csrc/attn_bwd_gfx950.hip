@@ -791,6 +791,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
     const int st = validate_bwd(d);
     if (st != COSMOS_ATTN_OK) return st;
     if (!workspace || workspace_bytes < cosmos_attn_bwd_workspace_bytes(d) || !aligned16(workspace)) return COSMOS_ATTN_WORKSPACE_TOO_SMALL;
+    if (!device_is_whole_mi355x()) return COSMOS_ATTN_WRONG_DEVICE;
     hipStream_t stream = (hipStream_t)stream_;
     const BwdGeom g(d);
     const bool bf16 = d->dtype == COSMOS_ATTN_BF16;

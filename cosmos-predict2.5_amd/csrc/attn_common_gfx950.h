@@ -39,6 +39,13 @@ constexpr int kFragBytes = 1024;   // one MFMA A-operand fragment: 64 lanes x 16
 // the accumulators, which otherwise runs in nearly every one of a sweep's first dozens of steps (in every step of a short
 // sweep), runs about once per sweep.
 constexpr float kMaxSlack = 6.0f;
+// With tangents H = p dS s is rounded to the 16-bit type as well, and fp16 has the range for |dS s| up to 65504 only while
+// p <= 1 (the reference's range, flash_attention_jvp_triton.py:114,141); a p of up to 2^6 would overflow from |dS s| ~ 1e3 on.
+// So fp16 with tangents keeps the exact running max; bf16 (8 exponent bits) and the forward-only kernels use the slack.
+template <typename T>
+__device__ __host__ constexpr float max_slack_of(bool with_tangents) {
+    return (with_tangents && __is_same(T, _Float16)) ? 0.0f : kMaxSlack;
+}
 #ifndef COSMOS_ATTN_PREFETCH_GROUPS
 #define COSMOS_ATTN_PREFETCH_GROUPS 2   // LDS operand fetches run this many MFMA groups ahead of use
 #endif
@@ -118,6 +125,23 @@ inline int choose_splits(int rem, int n_steps) {
         if (cost < best_cost - 1e-9) { best_cost = cost; best = S; }
     }
     return best_cost <= 0.9 ? best : 1;
+}
+
+// The workgroup-to-XCD maps and the rounds-of-kNumCUs arithmetic of the attention kernels assume a whole MI355X (256 compute
+// units).  A partitioned device (CPX / DPX modes) reports fewer and would silently get wrong piece maps: looked up once per
+// device ordinal, refused with a status code.  (Needs <mutex>.)
+inline bool device_is_whole_mi355x() {
+    static std::mutex mu;
+    static signed char state[64] = {};   // 0 = not looked up, 1 = yes, -1 = no
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return false; }
+    std::lock_guard<std::mutex> lock(mu);
+    if (state[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) { (void)hipGetLastError(); return false; }
+        state[dev] = n == kNumCUs ? 1 : -1;
+    }
+    return state[dev] == 1;
 }
 
 inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }

@@ -46,6 +46,7 @@
 #include <stddef.h>
 #include <stdlib.h>
 
+#include <atomic>
 #include <mutex>
 #include <set>
 #include <type_traits>
@@ -238,7 +239,7 @@ struct ScoreWave {
         }
         const float m_new = fmaxf(m_run, mx * scale_log2);
         float alpha = 1.0f;
-        if (__any(m_new > m_run + kMaxSlack)) {
+        if (__any(m_new > m_run + max_slack_of<T>(JVP))) {
             alpha = __builtin_amdgcn_exp2f(m_run - m_new);
             l_run *= alpha;
             r_run *= alpha;
@@ -1540,23 +1541,24 @@ SplitPlan plan_split(const cosmos_attn_desc* d) {
 // Short key sequences go to attn_qstream_kernel: number of workgroups (0 = use the other kernels).  The kernel cuts the
 // line of (query block, head) pairs into pieces of equal weight itself, so the launch is a small multiple of the number
 // of compute units (every unit gets the same number of equal pieces); it pays from a few blocks per workgroup on.
-// COSMOS_ATTN_STREAM_CHUNK (blocks per workgroup; 1 = off) overrides the choice: tuning and tests.
+// cosmos_attn_set_stream_override() replaces the choice (tuning and tests); nothing in the per-call path reads the environment.
 constexpr int kStreamMaxTiles = 64;       // up to 2048 keys
 constexpr int kStreamGroupsPerCU = 1;       // one workgroup fills a compute unit (8 wavefronts, 2 per SIMD at 256 registers): a single round
 constexpr int kStreamMinPairs = 1024;     // four blocks per workgroup: from there on the stream is faster than one workgroup per block (measured)
+std::atomic<int> g_stream_chunk{0};       // query blocks per workgroup (1 = never stream), 0 = the library's own choice
+std::atomic<int> g_stream_groups{0};      // number of workgroups, 0 = the library's own choice
 int stream_groups_of(const cosmos_attn_desc* d) {
     if (d->causal || d->d_qk != d->d_v || n_tiles_of(d) > kStreamMaxTiles) return 0;
     // the kernel addresses q and o inside a head with 32-bit byte offsets
     if ((int64_t)d->Lq * d->q_stride[2] >= ((int64_t)1 << 30) || (int64_t)d->Lq * d->o_stride[2] >= ((int64_t)1 << 30)) return 0;
     const int n_qt = (d->Lq + kBlockM - 1) / kBlockM;
     const int64_t pairs = (int64_t)n_qt * d->B * d->H;
-    if (const char* e = getenv("COSMOS_ATTN_STREAM_CHUNK")) {
-        const int chunk = atoi(e);
+    if (const int chunk = g_stream_chunk.load(std::memory_order_relaxed)) {
         if (chunk < 2 || pairs < 2) return 0;
         const int64_t groups = ((pairs + chunk - 1) / chunk + 7) / 8 * 8;     // a multiple of the number of XCDs
         return groups > (1 << 30) ? 0 : (int)groups;
     }
-    if (const char* e = getenv("COSMOS_ATTN_STREAM_GROUPS")) return atoi(e) > 0 ? (atoi(e) + 7) / 8 * 8 : 0;
+    if (const int groups = g_stream_groups.load(std::memory_order_relaxed)) return (groups + 7) / 8 * 8;
     return pairs >= kStreamMinPairs ? kNumCUs * kStreamGroupsPerCU : 0;
 }
 // LDS of attn_qstream_kernel: the layout of attn_fwd_jvp_kernel (AttnCfg::LDS_BYTES) + the per-block statistics slots
@@ -1617,12 +1619,18 @@ COSMOS_ATTN_API const char* cosmos_attn_status_string(int status) {
         case COSMOS_ATTN_BAD_ARG: return "bad argument (null pointer, non-positive size, ABI version, or tangent set other than none / q only / q,k,v)";
         case COSMOS_ATTN_BAD_SHAPE: return "bad shape (head dims must be in {16,32,64,128,256}; causal needs Lq == Lkv)";
         case COSMOS_ATTN_BAD_STRIDE: return "bad stride or alignment (16-byte aligned bases, strides multiple of 8 elements, innermost stride 1)";
-        case COSMOS_ATTN_UNSUPPORTED: return "unsupported dtype or head dim (bf16/fp16; backward and RMSNorm + RoPE: head dim <= 128)";
+        case COSMOS_ATTN_UNSUPPORTED: return "unsupported dtype or head dim (bf16/fp16 only)";
         case COSMOS_ATTN_WORKSPACE_TOO_SMALL: return "workspace too small or null";
         case COSMOS_ATTN_LAUNCH_FAILED: return "kernel launch failed";
+        case COSMOS_ATTN_WRONG_DEVICE: return "the current device is not a whole MI355X (gfx950 with 256 compute units in 8 XCDs): the kernels' workgroup-to-XCD maps assume it";
         case COSMOS_ATTN_STATIC_SCRATCH_EXCEEDED: return "problem needs more workspace than the library's static scratch array holds (cosmos_attn_static_scratch_bytes); use cosmos_attn_fwd_jvp with a caller-provided workspace";
         default: return "unknown status";
     }
+}
+
+COSMOS_ATTN_API void cosmos_attn_set_stream_override(int blocks_per_workgroup, int workgroups) {
+    g_stream_chunk.store(blocks_per_workgroup > 0 ? blocks_per_workgroup : 0, std::memory_order_relaxed);
+    g_stream_groups.store(workgroups > 0 ? workgroups : 0, std::memory_order_relaxed);
 }
 
 COSMOS_ATTN_API size_t cosmos_attn_workspace_bytes(const cosmos_attn_desc* d) {
@@ -1689,6 +1697,7 @@ int run_impl(const cosmos_attn_desc* d, const void* workspace, size_t workspace_
     // the two-stage run never cuts key ranges: it needs the image only
     const size_t need = scratch ? cosmos_attn_workspace_bytes(d) : align256(tiles_bytes_of(d));
     if (!workspace || workspace_bytes < need || !aligned16(workspace)) return COSMOS_ATTN_WORKSPACE_TOO_SMALL;
+    if (!device_is_whole_mi355x()) return COSMOS_ATTN_WRONG_DEVICE;
     const int mode = mode_of(d);
     if (is_wide(d)) return run_wide(d, workspace, stream);
     attn_kernel_t fn = d->dtype == COSMOS_ATTN_BF16 ? pick_dqk<__bf16>(d->d_qk, d->d_v, mode)

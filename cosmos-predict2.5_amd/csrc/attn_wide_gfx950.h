@@ -96,7 +96,7 @@ __global__ void __launch_bounds__(64 * kWideWaves) attn_wide_kernel(const AttnPa
         float lo, hi;
         both_halves(mx, lo, hi);
         const float m_new = fmaxf(m_run, fmaxf(lo, hi) * p.scale_log2);
-        if (__any(m_new > m_run + kMaxSlack)) {
+        if (__any(m_new > m_run + max_slack_of<T>(JVP))) {
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
             l_run *= alpha;
             r_run *= alpha;

@@ -156,15 +156,21 @@ class Attention(nn.Module):
         is reused only for the very same tensor object (held by a weak reference, so a new tensor that happens to get the
         freed one's address is never mistaken for it) at the same version, with weights at the same address and version."""
         params = (k_proj.weight, k_norm.weight, v_proj.weight)
-        key = (context._version, tuple(context.shape), context.dtype, context.device,
-               tuple((w.data_ptr(), w._version, w.dtype) for w in params))
-        hit = self._context_cache.get(slot) if self.cache_context else None
-        if hit is not None and hit[0]() is context and hit[1] == key:
-            return hit[2]
+        # Inference tensors (made under torch.inference_mode(), as the reference's text encoder makes the context) carry no
+        # version counter, so a change in place could not be noticed: those are re-tiled on every call.
+        cacheable = self.cache_context and not (context.is_inference() or any(w.is_inference() for w in params))
+        key = None
+        if cacheable:
+            compute_dtype = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled("cuda") else k_proj.weight.dtype
+            key = (context._version, tuple(context.shape), context.dtype, context.device, compute_dtype,
+                   tuple((w.data_ptr(), w._version, w.dtype) for w in params))
+            hit = self._context_cache.get(slot)
+            if hit is not None and hit[0]() is context and hit[1] == key:
+                return hit[2]
         k, _ = self._norm_rope(self._heads(k_proj(context)), k_norm, None)
         v = self._heads(v_proj(context))
         packed = ops.pack_kv(k.transpose(1, 2), v.transpose(1, 2))
-        if self.cache_context:
+        if cacheable:
             self._context_cache[slot] = (weakref.ref(context), key, packed)
         return packed
 
@@ -174,8 +180,12 @@ class Attention(nn.Module):
         return state
 
     def _context_is_fixed(self, x: torch.Tensor, context) -> bool:
-        return (context is not None) and isinstance(context, torch.Tensor) and x.is_cuda and not torch.is_grad_enabled() \
-            and isinstance(self.v_norm, nn.Identity) and not results_are_kept()
+        if context is None or not isinstance(context, torch.Tensor) or not x.is_cuda:
+            return False
+        if not isinstance(self.v_norm, nn.Identity) or results_are_kept():
+            return False
+        # no autograd graph will be built: grad mode off, or nothing on the way requires a gradient
+        return not (torch.is_grad_enabled() and (x.requires_grad or context.requires_grad or any(p.requires_grad for p in self.parameters())))
 
     # ------------------------------------------------------------------ the reference's surface
     def compute_qkv(self, x, context=None, rope_emb=None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:

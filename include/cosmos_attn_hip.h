@@ -40,7 +40,9 @@ enum cosmos_attn_status {
     COSMOS_ATTN_UNSUPPORTED = 4,    /* dtype / head-dim combination not built */
     COSMOS_ATTN_WORKSPACE_TOO_SMALL = 5,
     COSMOS_ATTN_LAUNCH_FAILED = 6,  /* hipGetLastError() != hipSuccess after a launch */
-    COSMOS_ATTN_STATIC_SCRATCH_EXCEEDED = 7   /* cosmos_attn_fwd_jvp_static: workspace need > COSMOS_ATTN_STATIC_SCRATCH_BYTES */
+    COSMOS_ATTN_STATIC_SCRATCH_EXCEEDED = 7,  /* cosmos_attn_fwd_jvp_static: workspace need > COSMOS_ATTN_STATIC_SCRATCH_BYTES */
+    COSMOS_ATTN_WRONG_DEVICE = 8    /* the current device does not report 256 compute units (a partitioned MI355X, another part):
+                                       checked once per device at the first attention launch */
 };
 
 /* size of the static device array behind cosmos_attn_fwd_jvp_static (64 MiB) */
@@ -83,6 +85,15 @@ COSMOS_ATTN_API int cosmos_attn_abi_version(void);
 
 /* Human-readable text for a status code (static storage). */
 COSMOS_ATTN_API const char *cosmos_attn_status_string(int status);
+
+/*
+ * Tuning and test hook, process-wide; no counterpart in the reference.  Short key sequences (text cross-attention) are
+ * served by a kernel that streams consecutive query blocks through one workgroup; the library chooses when and with how
+ * many workgroups.  blocks_per_workgroup > 1 forces that kernel with that many query blocks per workgroup, 1 turns it off,
+ * 0 leaves the choice to the library; workgroups > 0 (used when blocks_per_workgroup is 0) sets the number of workgroups
+ * directly.  (0, 0) restores the default.  Nothing in the per-call path reads the environment.
+ */
+COSMOS_ATTN_API void cosmos_attn_set_stream_override(int blocks_per_workgroup, int workgroups);
 
 /*
  * Bytes of device workspace the call needs (K, V and their tangents re-tiled into the

@@ -354,6 +354,37 @@ def rows_oracle(q_rows, k, v, tq_rows=None, tk=None, tv=None, sm_scale=None, kv_
     return O, dO, lse
 
 
+def grads_rows_oracle(q_rows, k, v, dout_rows, sm_scale=None):
+    """dQ of a block of query rows, fp32 torch on CPU: a row of dQ depends on its own q and dout rows and on the full K, V
+    only (P, O, dP, D, dS of that row; closed form of ``grads_closed_form``).  q_rows, dout_rows: [..., R, d]; k, v:
+    [..., Lkv, d].  How the backward is checked at L=84480 (pinned against ``grads_closed_form`` in tests/test_oracle.py)."""
+    import torch
+
+    f32 = lambda x: x.detach().to("cpu", torch.float32)
+    q_rows, k, v, dout_rows = (f32(x) for x in (q_rows, k, v, dout_rows))
+    s = (1.0 / math.sqrt(q_rows.shape[-1])) if sm_scale is None else float(sm_scale)
+    P = torch.softmax((q_rows @ k.transpose(-1, -2)) * s, dim=-1)
+    O = P @ v
+    dP = dout_rows @ v.transpose(-1, -2)
+    dS = P * (dP - (dout_rows * O).sum(-1, keepdim=True))
+    return (dS @ k) * s
+
+
+def grads_cols_oracle(q, k_cols, v_cols, o, lse, dout, sm_scale=None):
+    """(dK, dV) of a block of keys, fp32 torch on CPU, given the forward's results as the backward itself is given them
+    (``o`` [..., Lq, d] and the natural-log ``lse`` [..., Lq] of the scaled scores over ALL keys): with them the columns
+    P[:, C] = exp(q k_C^T s - lse) need no other key, so dV_C = P_C^T dO and dK_C = s (P_C * (dO v_C^T - D))^T Q cost
+    Lq * |C| * d.  q, o, dout: [..., Lq, d]; k_cols, v_cols: [..., C, d].  Pinned against ``grads_closed_form``."""
+    import torch
+
+    f32 = lambda x: x.detach().to("cpu", torch.float32)
+    q, k_cols, v_cols, o, lse, dout = (f32(x) for x in (q, k_cols, v_cols, o, lse, dout))
+    s = (1.0 / math.sqrt(q.shape[-1])) if sm_scale is None else float(sm_scale)
+    P = torch.exp((q @ k_cols.transpose(-1, -2)) * s - lse[..., None])
+    dS = P * (dout @ v_cols.transpose(-1, -2) - (dout * o).sum(-1, keepdim=True))
+    return (dS.transpose(-1, -2) @ q) * s, P.transpose(-1, -2) @ dout
+
+
 # --------------------------------------------------------------------------- #
 # error metrics and synthetic inputs shared by tests / bench / smoke
 # --------------------------------------------------------------------------- #

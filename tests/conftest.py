@@ -51,3 +51,16 @@ def gpu():
 
     assert torch.cuda.is_available(), "GPU tests need a GPU"
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def stream_override(pkg):
+    """``stream_override(chunk=..., groups=...)`` steers short key sequences to (or away from) the query-streaming kernels through the
+    library's own hook ``cosmos_attn_set_stream_override``; the library's choice is restored after the test."""
+    lib = pkg._lib.load_library()
+
+    def set_(chunk=0, groups=0):
+        lib.cosmos_attn_set_stream_override(int(chunk), int(groups))
+
+    yield set_
+    lib.cosmos_attn_set_stream_override(0, 0)

@@ -198,3 +198,64 @@ def test_fixed_context_is_packed_once_and_reused(pkg, gpu, monkeypatch):
     xg = x.clone().requires_grad_(True)
     m(xg, other).float().sum().backward()
     assert len(calls) == n and xg.grad is not None
+
+
+def test_context_made_in_inference_mode(pkg, gpu):
+    """The reference makes the text context under ``torch.inference_mode()`` (inference/get_t5_emb.py:50): such tensors have
+    no version counter, so the module re-tiles them per call instead of caching, and gives the same bits as with the cache off."""
+    import copy
+    m = build(pkg, gpu, 256, 96, 2, 128, torch.bfloat16, seed=5)
+    ref = copy.deepcopy(m)
+    ref.cache_context = False
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(1, 200, 256, generator=g).to(gpu, torch.bfloat16)
+    tx = (torch.randn(1, 200, 256, generator=g) * 0.3).to(gpu, torch.bfloat16)
+    with torch.inference_mode():
+        context = torch.randn(1, 40, 96, generator=g).to(gpu, torch.bfloat16) * 1.0
+    assert context.is_inference()
+    for mode in (torch.no_grad, torch.inference_mode):
+        with mode():
+            a = m(x, context)
+            b = ref(x, context)
+        assert torch.equal(a, b)
+    a2, ta = m.forward_jvp(x, tx, context)
+    b2, tb = ref.forward_jvp(x, tx, context)
+    assert torch.equal(a2, b2) and torch.equal(ta, tb)
+    assert not m._context_cache                               # nothing was kept for the inference tensor
+
+
+def test_image_conditioned_cross_attention_cache_matches_uncached(pkg, gpu, monkeypatch):
+    """``I2VCrossAttention``: the packed text and image contexts (slots "text" and "image") are reused across forward and
+    forward mode, and the results equal those of the same module with the cache turned off; switching the autocast dtype
+    over the same context re-tiles instead of tripping on the cached image's dtype."""
+    import copy
+    torch.manual_seed(7)
+    m = pkg.I2VCrossAttention(256, 96, n_heads=2, head_dim=128, img_latent_dim=64)
+    m.init_weights()
+    m = m.to(device=gpu, dtype=torch.bfloat16).eval()
+    ref = copy.deepcopy(m)
+    ref.cache_context = False
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(2, 260, 256, generator=g).to(gpu, torch.bfloat16)
+    tx = (torch.randn(2, 260, 256, generator=g) * 0.3).to(gpu, torch.bfloat16)
+    ctx = (torch.randn(2, 48, 96, generator=g).to(gpu, torch.bfloat16), torch.randn(2, 20, 64, generator=g).to(gpu, torch.bfloat16))
+    calls = []
+    real_pack = pkg.ops.pack_kv
+    monkeypatch.setattr(pkg.ops, "pack_kv", lambda k, v: (calls.append(1), real_pack(k, v))[1])
+    with torch.no_grad():
+        a = m(x, ctx)
+    a2, ta = m.forward_jvp(x, tx, ctx)
+    assert len(calls) == 2                                    # text + image, packed once for both calls
+    with torch.no_grad():
+        b = ref(x, ctx)
+    b2, tb = ref.forward_jvp(x, tx, ctx)
+    assert len(calls) == 6
+    assert torch.equal(a, b) and torch.equal(a2, b2) and torch.equal(ta, tb)
+    n = len(calls)
+    mf = copy.deepcopy(m).float()                             # fp32 weights under two autocast dtypes over one context
+    cf = tuple(c.float() for c in ctx)
+    for dt in (torch.bfloat16, torch.float16, torch.bfloat16):
+        with torch.no_grad(), torch.autocast("cuda", dtype=dt):
+            y = mf(x.float(), cf)
+        assert y.dtype == dt and torch.isfinite(y.float()).all()
+    assert len(calls) == n + 6

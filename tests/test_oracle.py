@@ -260,3 +260,22 @@ def test_grads_closed_form_matches_finite_differences(oracle):
             args_m = {"q": (xm, k, v), "k": (q, xm, v), "v": (q, k, xm)}[name]
             fd = (loss(*args_p) - loss(*args_m)) / (2 * eps)
             assert abs(fd - g[idx]) < 1e-6, (name, idx, fd, g[idx])
+
+
+def test_grads_rows_and_cols_oracles_match_closed_form(oracle):
+    """The row-block (dQ) and key-block (dK, dV) oracles used at L=84480 equal the full fp64 closed form on the rows / keys
+    they cover; the key-block oracle takes the forward's o and lse as inputs, as the backward kernels do."""
+    q, k, v, tq, _, _ = oracle.make_inputs((2, 2, 200, 32), (2, 2, 150, 32), seed=11, dtype=torch.float32)
+    dout = tq * 7.0
+    dq, dk, dv = oracle.grads_closed_form(q, k, v, dout, sm_scale=0.21)
+    o, _, lse = oracle.closed_form(q, k, v, sm_scale=0.21)
+    rows, cols = slice(40, 168), slice(90, 150)
+    got = oracle.grads_rows_oracle(q[:, :, rows], k, v, dout[:, :, rows], sm_scale=0.21)
+    assert oracle.error_metrics(got, dq[:, :, rows])[1] < 1e-5
+    gk, gv = oracle.grads_cols_oracle(q, k[:, :, cols], v[:, :, cols], torch.from_numpy(o), torch.from_numpy(lse), dout, sm_scale=0.21)
+    assert oracle.error_metrics(gk, dk[:, :, cols])[1] < 1e-5 and oracle.error_metrics(gv, dv[:, :, cols])[1] < 1e-5
+    # a wrong lse (e.g. base-2, or of unscaled scores) or a dropped D term must fail: the check has teeth
+    bad_k, bad_v = oracle.grads_cols_oracle(q, k[:, :, cols], v[:, :, cols], torch.from_numpy(o), torch.from_numpy(lse) * 1.4427, dout, sm_scale=0.21)
+    assert oracle.error_metrics(bad_v, dv[:, :, cols])[1] > 1e-2
+    bad_k, _ = oracle.grads_cols_oracle(q, k[:, :, cols], v[:, :, cols], torch.zeros_like(torch.from_numpy(o)), torch.from_numpy(lse), dout, sm_scale=0.21)
+    assert oracle.error_metrics(bad_k, dk[:, :, cols])[1] > 1e-2

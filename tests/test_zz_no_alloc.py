@@ -83,11 +83,11 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit(pkg, oracle, gpu):
     assert lib.cosmos_attn_fwd_jvp_static(ctypes.byref(D), None) == L.ST_BAD_ARG
 
 
-def test_static_scratch_entry_point_under_graph_capture(pkg, oracle, gpu, monkeypatch):
+def test_static_scratch_entry_point_under_graph_capture(pkg, oracle, gpu, stream_override):
     """What the entry point is for: a HIP graph captured around it (no allocation inside the capture: the outputs exist
     already), replayed with new input contents and eager work in between, matches eager calls bit for bit.  The streaming
     kernel is forced so that the capture holds the cross-attention path."""
-    monkeypatch.setenv("COSMOS_ATTN_STREAM_CHUNK", "3")
+    stream_override(chunk=3)
     L, lib = pkg._lib, pkg._lib.load_library()
     make = lambda seed: [x.to(gpu) for x in oracle.make_inputs((2, 2, 900, 128), (2, 2, 200, 128), seed=seed)[:4]]
     q, k, v, tq = make(0)
