@@ -66,7 +66,7 @@ class AttnBwdDesc(ctypes.Structure):
         ("d", ctypes.c_int32),
         ("causal", ctypes.c_int32),
         ("sm_scale", ctypes.c_float),
-        ("reserved", ctypes.c_int32),
+        ("max_ds_mib", ctypes.c_int32),
         ("q", ctypes.c_void_p),
         ("k", ctypes.c_void_p),
         ("v", ctypes.c_void_p),

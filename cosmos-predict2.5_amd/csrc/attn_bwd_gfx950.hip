@@ -184,13 +184,20 @@ struct BwdParams {
     // are cut into `splits` ranges of the stream, one workgroup each, which leave fp32 partial sums for bwd_combine_kernel
     int n_blk, n_full, n_rem, splits;
     float* part;                       // [(pair - n_full) * splits + split][kBlock][D] (dQ) or [..][kBlock][2][D] (dV, dK)
+    // A launch serves the heads [bh0, bh0 + pairs / n_blk) of the call (one group of heads at a time when dS is kept).
+    int bh0;
+    // dK/dV kernel with SPILL: every 32 x 32 tile of dS = P * (dP - D) it forms is also written, as the two 1 KB operand
+    // fragments the score wavefront hands over, to ds[local head][query tile][key tile] (2 KB each) for attn_dq_from_ds_kernel
+    char* ds;
+    int64_t ds_head_bytes;             // n_q_tiles * n_kt_pad * 2048
+    int n_kt_pad;                      // key tiles per query tile in `ds`: 4 * number of 128-key blocks
 };
 
 extern __shared__ __attribute__((aligned(1024))) char smem[];
 
 constexpr int kBwdSweepStagger = 2;   // tiles between the sweep starts of workgroups that share an L2 (3 as in the forward kernels: dQ kernel 1 % slower, 25 % more traffic)
 
-template <typename T, int D, int KIND>
+template <typename T, int D, int KIND, bool SPILL = false>
 struct BwdScoreWave {
     typedef BwdCfg<D, KIND> C;
     typedef typename VecOf<T>::v8 V8;
@@ -221,7 +228,7 @@ struct BwdScoreWave {
 
     // One step: elementwise work on the tile whose scores are in `x` (statistics fragment `stats` in the dK/dV
     // kernel) interleaved with the score MFMAs of the next tile (score-side part `spart`) into `xn`.
-    __device__ __forceinline__ void step(const Scores& x, Scores& xn, const char* spart, const char* stats, unsigned ph_out) {
+    __device__ __forceinline__ void step(const Scores& x, Scores& xn, const char* spart, const char* stats, unsigned ph_out, char* ds_dst = nullptr) {
         V8 uf[2], wf[2];
         V8 fa[NC], fb[NC];
         float l2v[16], ddv[16];
@@ -267,6 +274,10 @@ struct BwdScoreWave {
         } else {
             asm volatile("ds_write_b128 %0, %1" ::"v"(pa), "v"(wf[0]) : "memory");
             asm volatile("ds_write_b128 %0, %1 offset:1024" ::"v"(pa), "v"(wf[1]) : "memory");
+        }
+        if (SPILL) {   // this lane's 2 x 16 bytes of the tile's dS (compiler-generated stores: it knows their data hazards)
+            __builtin_nontemporal_store(wf[0], reinterpret_cast<V8*>(ds_dst));
+            __builtin_nontemporal_store(wf[1], reinterpret_cast<V8*>(ds_dst + kFragBytes));
         }
     }
 
@@ -332,11 +343,12 @@ struct BwdOutputWave {
     }
 };
 
-template <typename T, int D, int KIND>
+template <typename T, int D, int KIND, bool SPILL = false>
 __global__ void __attribute__((amdgpu_flat_work_group_size(kBwdThreads, kBwdThreads), amdgpu_waves_per_eu(2, 2)))
 attn_bwd_kernel(const BwdParams p) {
+    static_assert(!SPILL || KIND == KIND_DKDV, "only the dK/dV kernel forms whole tiles of dS");
     typedef BwdCfg<D, KIND> C;
-    typedef BwdScoreWave<T, D, KIND> SW;
+    typedef BwdScoreWave<T, D, KIND, SPILL> SW;
     typedef BwdOutputWave<T, D, KIND> OW;
     typedef typename VecOf<T>::v8 V8;
     typedef typename VecOf<T>::v4 V4;
@@ -353,7 +365,7 @@ attn_bwd_kernel(const BwdParams p) {
     const bool partial = bid >= p.n_full && p.splits > 1;
     const int pair = partial ? p.n_full + (bid - p.n_full) / p.splits : bid;
     const int split = partial ? (bid - p.n_full) % p.splits : 0;
-    const int blk = pair % p.n_blk, bh = pair / p.n_blk, b = bh / p.H, h = bh % p.H;
+    const int blk = pair % p.n_blk, bhl = pair / p.n_blk, bh = p.bh0 + bhl, b = bh / p.H, h = bh % p.H;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const bool score_role = wave < 4;            // wavefronts w and w + 4 (same SIMD) serve stationary rows 32 w .. 32 w + 31
@@ -452,15 +464,20 @@ attn_bwd_kernel(const BwdParams p) {
         asm volatile("" ::: "memory");
         w.scores_plain(sc0, sring);
         if (n_steps > 0 && need_mask(tile_at(0))) mask(sc0, tile_at(0));
+        // where this wavefront pair's dS tiles go: [local head][stream tile][4 blk + qw], this lane's 16 bytes
+        char* const ds_lane = SPILL ? p.ds + (int64_t)bhl * p.ds_head_bytes + ((int64_t)(4 * blk + qw) * 2 * kFragBytes + lane * 16) : nullptr;
+        const int64_t ds_row = (int64_t)p.n_kt_pad * 2 * kFragBytes;
+        int t_c = tile_at(0);           // tile whose scores are `cur`
         auto body = [&](int s, typename SW::Scores& cur, typename SW::Scores& nxt) {
-            __builtin_amdgcn_s_waitcnt(0xC07F);   // own hand-over stores of step s-1 done
+            __builtin_amdgcn_s_waitcnt(0xC07F);   // own hand-over stores of step s-1 done (lgkmcnt(0); the dS stores to memory are not waited for)
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             if (s < n_steps) {
                 w.step(cur, nxt, sring + ((s + 1) % kRingS) * SP_BYTES, string + (s % kRingStats) * kFragBytes,
-                       lds0 + ph_base + (s & 1) * 4 * C::PH_BYTES);
+                       lds0 + ph_base + (s & 1) * 4 * C::PH_BYTES, SPILL ? ds_lane + t_c * ds_row : nullptr);
                 if (s + 1 < n_steps && need_mask(t_o)) mask(nxt, t_o);
             }
+            t_c = wrap_inc(t_c);
             t_o = wrap_inc(t_o);   // tile at sweep position s + 2
         };
         for (int s = 0; s <= n_steps; s += 2) {
@@ -670,7 +687,7 @@ __global__ void __launch_bounds__(256) bwd_combine_kernel(const BwdParams p, int
     const int c = (threadIdx.x % tpr) * 4;
     const int pair_i = (int)(r / kBlock), wrow = (int)(r % kBlock);
     const int pair = p.n_full + pair_i;
-    const int blk = pair % p.n_blk, bh = pair / p.n_blk, b = bh / p.H, h = bh % p.H;
+    const int blk = pair % p.n_blk, bh = p.bh0 + pair / p.n_blk, b = bh / p.H, h = bh % p.H;
     const int row = blk * kBlock + wrow;
     if (pair_i >= p.n_rem || row >= p.L_stat) return;
     const int W = DKDV ? 2 * D : D;
@@ -695,8 +712,168 @@ __global__ void __launch_bounds__(256) bwd_combine_kernel(const BwdParams p, int
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------- dQ from kept dS
+// When the dK/dV kernel keeps its 16-bit dS tiles, dQ = s dS K is one product per tile instead of three (no second
+// computation of S and dP): a pass that streams dS from memory once and is bound by that stream (2 bytes per score
+// element; K^T comes from the L2).  A workgroup owns 256 queries, one 32-query tile per wavefront (8 wavefronts, two per
+// SIMD); per 32-key step a wavefront copies its own 2 KB dS tile and an eighth of the shared 32-key K^T part into an LDS
+// ring with direct-to-LDS loads kDsRing - 1 steps ahead, and accumulates dQ^T += K^T W with W = dS^T.
+// A dS tile lies in memory as the dK/dV kernel's score wavefront held it -- lane = key, eight queries per 16 bytes -- and is
+// wanted with lane = query, eight keys per lane: the transposing LDS read (ds_read_b64_tr_b16) does that.  Within a
+// group of 16 lanes, lane i passes the address of 8 bytes (row i of a 16 x 4 matrix M of 16-bit values) and receives
+// M[i/4 + 4k][i%4], k = 0..3.  A row of M here is one key's dS for 4 consecutive queries, so lane (query, half hh) gets, for
+// key chunk c and read t, the keys 16 c + 8 t + 4 hh + k -- the order in which a V^T-type fragment of K^T holds them.
+constexpr int kDsRing = 6;            // steps of dS / K^T in flight per workgroup
+constexpr int kDqWaves = 8;           // query tiles per workgroup
+constexpr int kDqThreads = 64 * kDqWaves;
+
+struct DqFromDsParams {
+    const char* ds;                    // [local head][n_q_tiles][n_kt_pad][2 KB]
+    int64_t ds_head_bytes;
+    int n_kt_pad;
+    const char* kt_img;                // K^T stream: [B*H][n_k_tiles][2 NDB fragments]
+    void* dq;
+    int64_t o_sb, o_sh, o_sl;
+    int H, Lq, Lkv, n_q_tiles, n_k_tiles, n_blk, bh0, causal;
+    float sm_scale;
+};
+
+template <int D>
+struct DqCfg {
+    static constexpr int NDB = (D + 31) / 32;
+    static constexpr int KT_FR = 2 * NDB, KT_BYTES = KT_FR * kFragBytes;
+    static constexpr int W_BYTES = 2 * kFragBytes;                       // one dS tile
+    static constexpr int SLOT_BYTES = kDqWaves * W_BYTES + KT_BYTES;
+    static constexpr int LDS_BYTES = kDsRing * SLOT_BYTES;
+    static constexpr int LOADS = 3;                                      // per wavefront per step: 2 (dS tile) + 1 (K^T fragment)
+};
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+template <typename T, int D>
+__global__ void __attribute__((amdgpu_flat_work_group_size(kDqThreads, kDqThreads), amdgpu_waves_per_eu(2, 2)))
+attn_dq_from_ds_kernel(const DqFromDsParams p) {
+    typedef DqCfg<D> C;
+    typedef typename VecOf<T>::v8 V8;
+    typedef typename VecOf<T>::v4 V4;
+    constexpr int NDB = C::NDB;
+    // vmcnt(n): the loads of the newest kDsRing - 2 steps may still be in flight
+    constexpr int IN_FLIGHT = C::LOADS * (kDsRing - 2);
+    constexpr int WAIT_LOADS = (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14) | 0x0F70;
+
+    const int blk = blockIdx.x % p.n_blk, bhl = blockIdx.x / p.n_blk, bh = p.bh0 + bhl, b = bh / p.H, h = bh % p.H;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 31, hh = lane >> 5;
+    const int qt = blk * kDqWaves + wave;          // this wavefront's query tile
+    const bool live_tile = qt < p.n_q_tiles;
+    const int row = qt * kRows + j;
+
+    // key tiles this workgroup walks: all, or up to its last query's diagonal when causal
+    int n_steps = p.n_k_tiles;
+    if (p.causal) { const int lim = blk * kDqWaves + kDqWaves; n_steps = n_steps < lim ? n_steps : lim; }
+
+    // this wavefront's run of dS tiles (one query tile, all key tiles: contiguous), and the head's K^T stream
+    const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(p.ds) + (int64_t)bhl * p.ds_head_bytes + (int64_t)(live_tile ? qt : 0) * p.n_kt_pad * C::W_BYTES, 0,
+        live_tile ? p.n_kt_pad * C::W_BYTES : 0, 0x00020000);   // no tile: every load returns zeros
+    const __amdgpu_buffer_rsrc_t rs_k = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(p.kt_img) + (size_t)bh * p.n_k_tiles * C::KT_BYTES, 0, p.n_k_tiles * C::KT_BYTES, 0x00020000);
+    const int kfrag = wave % C::KT_FR;             // the K^T fragment this wavefront copies (copied redundantly when there are fewer than 8)
+    auto issue = [&](int u) {                      // loads of sweep position u (clamped: positions past the end repeat the last tile, unused)
+        const int t = __builtin_amdgcn_readfirstlane(u < n_steps ? u : n_steps - 1);
+        char* slot = smem + (u % kDsRing) * C::SLOT_BYTES;
+        issue_part<2>(rs_w, slot + wave * C::W_BYTES, lane * 16, t * C::W_BYTES);
+        lds_load<0>(rs_k, slot + kDqWaves * C::W_BYTES + kfrag * kFragBytes, lane * 16, t * C::KT_BYTES + kfrag * kFragBytes);
+    };
+#pragma unroll
+    for (int u = 0; u < kDsRing - 1; ++u) issue(u);
+
+    f32x16 acc[NDB];
+#pragma unroll
+    for (int i = 0; i < NDB; ++i) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+    }
+    // transposing read: byte offset, inside a dS tile, of the 8 bytes this lane passes for key chunk 0, read 0
+    //   group g = lane / 16: queries 16 (g % 2) .. + 15, key half g / 2;  lane i of the group passes row r = i:
+    //   queries 16 (g%2) + 4 (r%4) .. + 3 of key 4 (g/2) + r/4  (+ 16 c + 8 t).  In the tile: fragment g%2 (queries 16 (g%2) ..),
+    //   lane index key + 32 (r%2), second 8 bytes of the lane's 16 when (r%4)/2.
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;   // LDS address of smem[0]
+    const int g16 = lane >> 4, r16 = lane & 15;
+    const unsigned tr_off = (unsigned)((g16 & 1) * kFragBytes + (4 * (g16 >> 1) + (r16 >> 2) + 32 * (r16 & 1)) * 16 + 8 * ((r16 & 3) >> 1));
+
+    for (int s = 0; s < n_steps; ++s) {
+        __builtin_amdgcn_s_waitcnt(WAIT_LOADS);
+        __builtin_amdgcn_s_barrier();          // everybody's loads of step s have landed, everybody is done reading step s - 1
+        asm volatile("" ::: "memory");
+        issue(s + kDsRing - 1);                // into the slot of step s - 1
+        const char* slot = smem + (s % kDsRing) * C::SLOT_BYTES;
+        // (written out: the compiler takes the builtin of this read for an access that may alias the direct-to-LDS loads in
+        // flight and puts vmcnt(0) in front of it, which would end the prefetch; it does not see through the asm, so the
+        // wait for the four results is in the block as well)
+        const unsigned wt = lds0 + (unsigned)((s % kDsRing) * C::SLOT_BYTES + wave * C::W_BYTES) + tr_off;
+        s16x4 t00, t01, t10, t11;
+        asm volatile("ds_read_b64_tr_b16 %0, %4\n\t"
+                     "ds_read_b64_tr_b16 %1, %4 offset:128\n\t"
+                     "ds_read_b64_tr_b16 %2, %4 offset:256\n\t"
+                     "ds_read_b64_tr_b16 %3, %4 offset:384\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&v"(t00), "=&v"(t01), "=&v"(t10), "=&v"(t11) : "v"(wt) : "memory");
+        V8 wf[2];
+        wf[0] = __builtin_shufflevector(__builtin_bit_cast(V4, t00), __builtin_bit_cast(V4, t01), 0, 1, 2, 3, 4, 5, 6, 7);
+        wf[1] = __builtin_shufflevector(__builtin_bit_cast(V4, t10), __builtin_bit_cast(V4, t11), 0, 1, 2, 3, 4, 5, 6, 7);
+        // dead operands become zeros: tiles the (causal) dK/dV kernel never formed, keys past the end of the last tile
+        const bool unformed = p.causal && (s / 4) * 4 > qt;
+        if (unformed || !live_tile || s * kRows + kRows > p.Lkv) {
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int key = s * kRows + 16 * c + 8 * (e >> 2) + 4 * hh + (e & 3);
+                    if (unformed || !live_tile || key >= p.Lkv) wf[c][e] = (T)0.0f;
+                }
+            }
+        }
+        const char* kt = slot + kDqWaves * C::W_BYTES + lane * 16;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+                acc[db] = mfma32(*reinterpret_cast<const V8*>(kt + (2 * db + c) * kFragBytes), wf[c], acc[db]);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);        // drain the trailing loads before the LDS is released
+    if (live_tile && row < p.Lq) {
+        T* o1 = reinterpret_cast<T*>(p.dq) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)row * p.o_sl;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = 32 * db + 8 * g + 4 * hh;   // registers 4g..4g+3 are 4 consecutive channels
+                if (d < D) {
+                    V4 v1;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v1[r] = (T)(acc[db][4 * g + r] * p.sm_scale);
+                    *reinterpret_cast<V4*>(o1 + d) = v1;
+                }
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ host
 typedef void (*bwd_kernel_t)(const BwdParams);
+
+typedef void (*dq_from_ds_kernel_t)(const DqFromDsParams);
+
+// Keeping dS pays where the two products it saves are large next to the 4 bytes per score element it moves: head dim 128.
+inline bool spill_head_dim(int d) { return d == 128; }
+template <typename T>
+bwd_kernel_t pick_dkdv_spill(int d) { return d == 128 ? attn_bwd_kernel<T, 128, KIND_DKDV, true> : nullptr; }
+template <typename T>
+dq_from_ds_kernel_t pick_dq_from_ds(int d) { return d == 128 ? attn_dq_from_ds_kernel<T, 128> : nullptr; }
 
 template <typename T, int KIND>
 bwd_kernel_t pick_bwd(int d) {
@@ -734,12 +911,35 @@ struct BwdGeom {
             part_bytes = 0;
             return;
         }
-        dkdv = plan((d->Lkv + kBlock - 1) / kBlock, (int)bh, n_q_tiles, d->causal != 0);
+        const int n_kblk = (d->Lkv + kBlock - 1) / kBlock;
+        // Keep dS?  Its tiles for one head take n_q_tiles * n_kt_pad * 2 KB; heads are served in groups that fit the budget
+        // (desc->max_ds_mib: 0 = kDefaultDsMiB, > 0 = that many MiB, < 0 = never keep dS).
+        n_kt_pad = 4 * n_kblk;
+        ds_head_bytes = (size_t)n_q_tiles * n_kt_pad * 2 * kFragBytes;
+        const int64_t budget = d->max_ds_mib < 0 ? 0 : (int64_t)(d->max_ds_mib > 0 ? d->max_ds_mib : kDefaultDsMiB) << 20;
+        if (spill_head_dim(d->d) && (int64_t)ds_head_bytes <= budget && (int64_t)n_kt_pad * 2 * kFragBytes < ((int64_t)1 << 31)) {
+            spill = true;
+            const int64_t fit = budget / (int64_t)ds_head_bytes;
+            group = (int)(fit < (int64_t)bh ? fit : (int64_t)bh);
+            ds_bytes = (size_t)group * ds_head_bytes;
+            k_tile_bytes = (size_t)(2 * ndb) * kFragBytes;            // the key stream holds K^T alone
+            k_img_bytes = bh * n_k_tiles * k_tile_bytes;
+        }
+        dkdv = plan(n_kblk, spill ? group : (int)bh, n_q_tiles, d->causal != 0);
         dq = plan((d->Lq + kBlock - 1) / kBlock, (int)bh, n_k_tiles, d->causal != 0);
-        const size_t p1 = (size_t)dkdv.n_rem * dkdv.splits * kBlock * 2 * d->d * sizeof(float);
-        const size_t p2 = (size_t)dq.n_rem * dq.splits * kBlock * d->d * sizeof(float);
+        size_t p1 = (size_t)dkdv.n_rem * dkdv.splits * kBlock * 2 * d->d * sizeof(float);
+        if (spill && bh % group) {   // the last, smaller group has a plan of its own
+            const Plan last = plan(n_kblk, (int)(bh % group), n_q_tiles, d->causal != 0);
+            const size_t p3 = (size_t)last.n_rem * last.splits * kBlock * 2 * d->d * sizeof(float);
+            p1 = p1 > p3 ? p1 : p3;
+        }
+        const size_t p2 = spill ? 0 : (size_t)dq.n_rem * dq.splits * kBlock * d->d * sizeof(float);
         part_bytes = ((p1 > p2 ? p1 : p2) + 1023) / 1024 * 1024;     // the two kernels run one after the other
     }
+    static constexpr int kDefaultDsMiB = 32 * 1024;
+    bool spill = false;
+    int group = 0, n_kt_pad = 0;        // heads per group; key tiles per query tile in the dS buffer
+    size_t ds_head_bytes = 0, ds_bytes = 0;
     // How the (block of stationary rows, head) pairs of a kernel are dealt out (see choose_splits): the pairs of a partly
     // filled last round of workgroups are cut along the stream and bwd_combine_kernel adds the ranges up.
     struct Plan { int n_blk, n_pairs, n_full, n_rem, splits; };
@@ -784,7 +984,7 @@ extern "C" {
 COSMOS_ATTN_API size_t cosmos_attn_bwd_workspace_bytes(const cosmos_attn_bwd_desc* d) {
     if (validate_bwd(d) != COSMOS_ATTN_OK) return 0;
     const BwdGeom g(d);
-    return g.stats_bytes + g.q_img_bytes + g.k_img_bytes + g.part_bytes;
+    return g.stats_bytes + g.q_img_bytes + g.k_img_bytes + g.part_bytes + g.ds_bytes;
 }
 
 COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspace, size_t workspace_bytes, void* stream_) {
@@ -804,6 +1004,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
     char* q_img = ws + g.stats_bytes;
     char* k_img = q_img + g.q_img_bytes;
     float* part = (float*)(k_img + g.k_img_bytes);
+    char* ds = (char*)part + g.part_bytes;
     const int BH = d->B * d->H;
     auto launch = [&](bwd_kernel_t fn, size_t lds, const BwdGeom::Plan& pl, BwdParams& bp, bool is_dkdv) {
         bp.n_blk = pl.n_blk; bp.n_full = pl.n_full; bp.n_rem = pl.n_rem; bp.splits = pl.splits; bp.part = part;
@@ -842,12 +1043,12 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
         pp.tile_frags = (int)(g.q_tile_bytes / kFragBytes);
         hipLaunchKernelGGL(pack_stream_kernel, dim3(g.n_q_tiles, BH), dim3(kPackThreads), 0, stream, pp);
     }
-    {   // key stream: K, V, K^T
+    {   // key stream: K, V, K^T  (K^T alone when dS is kept: the pass that reads it forms no scores)
         PackBwdParams pp;
         pp.a1 = src_of(d->k, d->k_stride); pp.a2 = src_of(d->v, d->v_stride);
         pp.c1 = src_of(d->k, d->k_stride); pp.c2 = PackSrc{nullptr, 0, 0, 0};
         pp.stats = nullptr; pp.out = (uint4*)k_img;
-        pp.H = d->H; pp.L = d->Lkv; pp.d = d->d; pp.n_tiles = g.n_k_tiles; pp.nc = g.nc; pp.ndb = g.ndb;
+        pp.H = d->H; pp.L = d->Lkv; pp.d = d->d; pp.n_tiles = g.n_k_tiles; pp.nc = g.spill ? 0 : g.nc; pp.ndb = g.ndb;
         pp.tile_frags = (int)(g.k_tile_bytes / kFragBytes);
         hipLaunchKernelGGL(pack_stream_kernel, dim3(g.n_k_tiles, BH), dim3(kPackThreads), 0, stream, pp);
     }
@@ -856,12 +1057,40 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
     BwdParams bp;
     bp.stats = stats; bp.H = d->H; bp.causal = d->causal;
     bp.sm_scale = d->sm_scale; bp.scale_log2 = d->sm_scale * 1.4426950408889634f;
-    {   // dK, dV: stationary keys, streamed queries
+    bp.bh0 = 0; bp.ds = nullptr; bp.ds_head_bytes = 0; bp.n_kt_pad = 0;
+    auto set_dkdv = [&]() {   // dK, dV: stationary keys, streamed queries
         bp.st1 = d->k; bp.s1_sb = d->k_stride[0]; bp.s1_sh = d->k_stride[1]; bp.s1_sl = d->k_stride[2];
         bp.st2 = d->v; bp.s2_sb = d->v_stride[0]; bp.s2_sh = d->v_stride[1]; bp.s2_sl = d->v_stride[2];
         bp.out1 = d->dv; bp.o1_sb = d->dv_stride[0]; bp.o1_sh = d->dv_stride[1]; bp.o1_sl = d->dv_stride[2];
         bp.out2 = d->dk; bp.o2_sb = d->dk_stride[0]; bp.o2_sh = d->dk_stride[1]; bp.o2_sl = d->dk_stride[2];
         bp.stream = q_img; bp.L_stat = d->Lkv; bp.L_stream = d->Lq; bp.n_tiles = g.n_q_tiles;
+    };
+    if (g.spill) {
+        // dS kept: per group of heads, the dK/dV kernel (which writes the group's dS tiles), then the pass that turns them into dQ
+        bwd_kernel_t k_spill = bf16 ? pick_dkdv_spill<__bf16>(d->d) : pick_dkdv_spill<_Float16>(d->d);
+        dq_from_ds_kernel_t k_ds = bf16 ? pick_dq_from_ds<__bf16>(d->d) : pick_dq_from_ds<_Float16>(d->d);
+        if (!k_spill || !k_ds) return COSMOS_ATTN_UNSUPPORTED;
+        const size_t lds_ds = (size_t)kDsRing * (kDqWaves * 2 * kFragBytes + 2 * g.ndb * kFragBytes);
+        if (!allow_lds((const void*)k_ds, lds_ds)) return COSMOS_ATTN_LAUNCH_FAILED;
+        set_dkdv();
+        bp.ds = ds; bp.ds_head_bytes = (int64_t)g.ds_head_bytes; bp.n_kt_pad = g.n_kt_pad;
+        DqFromDsParams qp;
+        qp.ds = ds; qp.ds_head_bytes = (int64_t)g.ds_head_bytes; qp.n_kt_pad = g.n_kt_pad; qp.kt_img = k_img;
+        qp.dq = d->dq; qp.o_sb = d->dq_stride[0]; qp.o_sh = d->dq_stride[1]; qp.o_sl = d->dq_stride[2];
+        qp.H = d->H; qp.Lq = d->Lq; qp.Lkv = d->Lkv; qp.n_q_tiles = g.n_q_tiles; qp.n_k_tiles = g.n_k_tiles;
+        qp.n_blk = (g.n_q_tiles + kDqWaves - 1) / kDqWaves; qp.causal = d->causal; qp.sm_scale = d->sm_scale;
+        for (int bh0 = 0; bh0 < BH; bh0 += g.group) {
+            const int heads = BH - bh0 < g.group ? BH - bh0 : g.group;
+            const BwdGeom::Plan pl = heads == g.group ? g.dkdv : BwdGeom::plan(g.dkdv.n_blk, heads, g.n_q_tiles, d->causal != 0);
+            bp.bh0 = bh0;
+            if (!launch(k_spill, g.lds_dkdv, pl, bp, true)) return COSMOS_ATTN_LAUNCH_FAILED;
+            qp.bh0 = bh0;
+            hipLaunchKernelGGL(k_ds, dim3((unsigned)(qp.n_blk * heads)), dim3(kDqThreads), lds_ds, stream, qp);
+        }
+        return hipGetLastError() == hipSuccess ? COSMOS_ATTN_OK : COSMOS_ATTN_LAUNCH_FAILED;
+    }
+    {
+        set_dkdv();
         if (!launch(k_dkdv, g.lds_dkdv, g.dkdv, bp, true)) return COSMOS_ATTN_LAUNCH_FAILED;
     }
     {   // dQ: stationary queries, streamed keys

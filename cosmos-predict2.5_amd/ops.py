@@ -251,11 +251,15 @@ def bwd(
     dout: torch.Tensor,
     causal: bool = False,
     sm_scale: Optional[float] = None,
+    max_ds_mib: Optional[int] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """(dq, dk, dv) for the cotangent ``dout`` of o; all tensors ``[B, H, L, d]`` views on one GPU, ``lse`` the
     forward's ``[B, H, Lq]`` fp32.  Mirrors the reference's ``_attention.backward``
     (cosmos_predict2/_src/predict2/utils/flash_attention_jvp_triton.py:505-561): equal head dims only (:507-509),
     outputs allocated like ``torch.empty_like`` of q, k, v (:513).
+
+    ``max_ds_mib``: workspace the call may spend on keeping the 16-bit dS tiles between its two passes (the descriptor's
+    field of that name; negative = never).  Default: 32 GiB, but no more than 40 % of the device memory free right now.
     """
     assert q.shape[-1] == k.shape[-1] and k.shape[-1] == v.shape[-1], "Backward not supported with different headdim."
     B, H, Lq, d = q.shape
@@ -287,7 +291,10 @@ def bwd(
     desc.B, desc.H, desc.Lq, desc.Lkv, desc.d = B, H, Lq, Lkv, d
     desc.causal = 1 if causal else 0
     desc.sm_scale = float(sm_scale)
-    desc.reserved = 0
+    if max_ds_mib is None:
+        free_bytes, _ = torch.cuda.mem_get_info(q.device)
+        max_ds_mib = max(1, min(32 * 1024, int(0.4 * free_bytes) >> 20))
+    desc.max_ds_mib = int(max_ds_mib)
     desc.q, desc.k, desc.v, desc.o, desc.dout = (x.data_ptr() for x in (q, k, v, o, dout))
     desc.lse = lse.data_ptr()
     desc.dq, desc.dk, desc.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()

@@ -156,7 +156,9 @@ typedef struct cosmos_attn_bwd_desc {
     int32_t d;               /* head dim of q, k and v, in {16,32,64,128,256} */
     int32_t causal;
     float sm_scale;          /* the forward's softmax scale (`ctx.sm_scale`, JVP:499) */
-    int32_t reserved;        /* 0 */
+    int32_t max_ds_mib;      /* workspace the call may spend on keeping the 16-bit dS tiles between its two passes, in MiB:
+                                0 = library default (32 GiB), > 0 = that many, < 0 = never keep dS (the smallest workspace;
+                                the scores are then computed a second time for dq).  Results are deterministic either way. */
 
     const void *q, *k, *v, *o, *dout;   /* device */
     const float *lse;        /* [B,H,Lq] fp32 contiguous, as written by the forward */

@@ -227,3 +227,37 @@ def test_bwd_more_than_2_31_elements(pkg, oracle, gpu):
             want_dk += (ds_blk.T @ qh[rr]) * d ** -0.5
         check(oracle, f"dv keys of (b={b}, h={h})", dv[b, h, keys], want_dv.cpu())
         check(oracle, f"dk keys of (b={b}, h={h})", dk[b, h, keys], want_dk.cpu())
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [((2, 5, 700, 128), None), ((1, 3, 333, 128), (1, 3, 517, 128)), ((1, 7, 1100, 128), (1, 7, 90, 128))])
+def test_bwd_kept_ds_groups_of_heads_match_the_recomputing_path(pkg, oracle, gpu, shape, causal):
+    """At head dim 128 the dK/dV kernel keeps its 16-bit dS tiles and dq comes from them in a second pass, heads served in groups
+    that fit ``max_ds_mib``.  A budget of a few MiB forces several groups (with a smaller last one); a negative one the path
+    that computes the scores twice.  All meet the oracle, agree with each other to rounding, and repeat bit for bit."""
+    shape_q, shape_kv = shape
+    if causal and shape_kv is not None:
+        pytest.skip("causal needs equal lengths")
+    q, k, v, _, _, _ = oracle.make_inputs(shape_q, shape_kv, seed=31)
+    g = torch.Generator().manual_seed(32)
+    dout = torch.randn(q.shape, generator=g).to(torch.bfloat16)
+    qd, kd, vd, dd = (x.to(gpu) for x in (q, k, v, dout))
+    o, _, lse = pkg.attention_with_lse(qd, kd, vd, causal=causal)
+    want = oracle.grads_closed_form(q, k, v, dout, causal=causal)
+    n_qt, n_kb = (q.shape[2] + 31) // 32, (k.shape[2] + 127) // 128
+    head_mib = n_qt * 4 * n_kb * 2048 / 2 ** 20
+    results = {}
+    for name, budget in (("recompute", -1), ("groups of 2", max(1, int(2 * head_mib + 0.999))), ("one group", 1024)):
+        print(f"  {name}: max_ds_mib={budget} (a head's dS: {head_mib:.2f} MiB)", flush=True)
+        got = pkg.ops.bwd(qd, kd, vd, o, lse, dd, causal=causal, max_ds_mib=budget)
+        again = pkg.ops.bwd(qd, kd, vd, o, lse, dd, causal=causal, max_ds_mib=budget)
+        torch.cuda.synchronize()
+        for nm, a, b, w in zip(("dq", "dk", "dv"), got, again, want):
+            assert torch.equal(a, b), f"{name}: {nm} differs between two calls"
+            check(oracle, f"{name} {nm}", a, w)
+        results[name] = got
+    # (the paths cut a thin last round of workgroups along the stream at different places, so their sums round differently:
+    # equal to rounding, not bit for bit)
+    for other in ("groups of 2", "one group"):
+        for a, b in zip(results[other], results["recompute"]):
+            assert (a.float() - b.float()).abs().max().item() <= 2e-2 * max(1.0, b.float().abs().max().item())

@@ -91,7 +91,7 @@ def test_status_codes_for_bad_descriptors(pkg):
 def good_bwd_desc(pkg, **over):
     D = pkg._lib.AttnBwdDesc()
     D.abi_version, D.dtype = pkg._lib.ABI_VERSION, pkg._lib.DTYPE_BF16
-    D.B, D.H, D.Lq, D.Lkv, D.d, D.causal, D.sm_scale, D.reserved = 1, 2, 100, 70, 64, 0, 0.1, 0
+    D.B, D.H, D.Lq, D.Lkv, D.d, D.causal, D.sm_scale, D.max_ds_mib = 1, 2, 100, 70, 64, 0, 0.1, 0
     fake = 0x7F0000000000  # never dereferenced: validation only looks at values
     for i, name in enumerate(("q", "k", "v", "o", "dout", "lse", "dq", "dk", "dv")):
         setattr(D, name, fake + 4096 * i)
