@@ -8,24 +8,27 @@
 // (cosmos_predict2/_src/predict2/utils/flash_attention_jvp_triton.py:505-561): same inputs (q, k, v, o, lse, dout),
 // same outputs (dq, dk, dv), gradient through O only, equal head dims required (:507-509).
 //
-// Two kernels with the structure of the forward kernel (warp-specialised, two wavefronts per SIMD: a "score"
-// wavefront that issues the QK^T-type MFMAs and the elementwise work, an "output" wavefront that owns the fp32
-// accumulators and issues the accumulating MFMAs; operands handed over through LDS; stream tiles of 32 rows
-// re-tiled once per call into 1 KB MFMA A-operand fragments and moved L2 -> LDS with direct-to-LDS loads):
+// Kernels with the structure of the forward kernel (wavefronts specialised by role, two per SIMD; operands handed over
+// through LDS; stream tiles of 32 rows re-tiled once per call into 1 KB MFMA A-operand fragments and moved L2 -> LDS with
+// direct-to-LDS loads):
 //   * dK/dV kernel: a workgroup owns 128 keys (K, V rows are the stationary B operands) and streams query tiles:
-//       S'^T-type scores  Sq = Q k^T,  dPq = dO v^T  (rows = streamed queries, columns = own keys),
+//       scores  Sq = Q k^T,  dPq = dO v^T  (rows = streamed queries, columns = own keys),
 //       U = P, W = dS as 16-bit B operands,   dV^T += dO^T U,   dK^T += Q^T W.
 //     LSE and D vary along the streamed rows; they travel with the stream as one extra fragment per tile.
-//   * dQ kernel: a workgroup owns 128 queries (Q, dO rows stationary) and streams key tiles:
-//       S^T = K q^T,  dP^T = V dO^T,   W = dS^T,   dQ^T += K^T W.      LSE and D are per-lane constants.
-// No atomics: results are bitwise reproducible.  P is recomputed in both kernels (7 matmuls instead of the
-// minimal 5).
+//     Head dim 128: attn_dkdv_quad_kernel (four roles per 64 keys, attn_bwd_quad_gfx950.h), which can also keep every dS tile
+//     in memory; other head dims: attn_bwd_kernel<T, D, KIND_DKDV> (score wavefront + output wavefront per 32 keys).
+//   * dQ from kept dS (head dim 128, when the workspace budget allows): attn_dq_from_ds_kernel streams the 16-bit dS tiles
+//     back once, dQ^T += K^T W with W = dS^T -- five matrix products per call in all, as the reference counts them.
+//   * dQ by recomputation (otherwise): attn_bwd_kernel<T, D, KIND_DQ>: a workgroup owns 128 queries (Q, dO rows stationary)
+//     and streams key tiles:  S^T = K q^T,  dP^T = V dO^T,   W = dS^T,   dQ^T += K^T W  (P computed a second time: seven products).
+// No atomics: results are bitwise reproducible.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stddef.h>
 
 #include <mutex>
 #include <set>
+#include <type_traits>
 #include <utility>
 
 #include "cosmos_attn_hip.h"
@@ -186,7 +189,7 @@ struct BwdParams {
     float* part;                       // [(pair - n_full) * splits + split][kBlock][D] (dQ) or [..][kBlock][2][D] (dV, dK)
     // A launch serves the heads [bh0, bh0 + pairs / n_blk) of the call (one group of heads at a time when dS is kept).
     int bh0;
-    // dK/dV kernel with SPILL: every 32 x 32 tile of dS = P * (dP - D) it forms is also written, as the two 1 KB operand
+    // dK/dV kernel that keeps dS: every 32 x 32 tile of dS = P * (dP - D) it forms is also written, as the two 1 KB operand
     // fragments the score wavefront hands over, to ds[local head][query tile][key tile] (2 KB each) for attn_dq_from_ds_kernel
     char* ds;
     int64_t ds_head_bytes;             // n_q_tiles * n_kt_pad * 2048
@@ -197,7 +200,7 @@ extern __shared__ __attribute__((aligned(1024))) char smem[];
 
 constexpr int kBwdSweepStagger = 2;   // tiles between the sweep starts of workgroups that share an L2 (3 as in the forward kernels: dQ kernel 1 % slower, 25 % more traffic)
 
-template <typename T, int D, int KIND, bool SPILL = false>
+template <typename T, int D, int KIND>
 struct BwdScoreWave {
     typedef BwdCfg<D, KIND> C;
     typedef typename VecOf<T>::v8 V8;
@@ -228,7 +231,7 @@ struct BwdScoreWave {
 
     // One step: elementwise work on the tile whose scores are in `x` (statistics fragment `stats` in the dK/dV
     // kernel) interleaved with the score MFMAs of the next tile (score-side part `spart`) into `xn`.
-    __device__ __forceinline__ void step(const Scores& x, Scores& xn, const char* spart, const char* stats, unsigned ph_out, char* ds_dst = nullptr) {
+    __device__ __forceinline__ void step(const Scores& x, Scores& xn, const char* spart, const char* stats, unsigned ph_out) {
         V8 uf[2], wf[2];
         V8 fa[NC], fb[NC];
         float l2v[16], ddv[16];
@@ -274,10 +277,6 @@ struct BwdScoreWave {
         } else {
             asm volatile("ds_write_b128 %0, %1" ::"v"(pa), "v"(wf[0]) : "memory");
             asm volatile("ds_write_b128 %0, %1 offset:1024" ::"v"(pa), "v"(wf[1]) : "memory");
-        }
-        if (SPILL) {   // this lane's 2 x 16 bytes of the tile's dS (compiler-generated stores: it knows their data hazards)
-            __builtin_nontemporal_store(wf[0], reinterpret_cast<V8*>(ds_dst));
-            __builtin_nontemporal_store(wf[1], reinterpret_cast<V8*>(ds_dst + kFragBytes));
         }
     }
 
@@ -343,12 +342,11 @@ struct BwdOutputWave {
     }
 };
 
-template <typename T, int D, int KIND, bool SPILL = false>
+template <typename T, int D, int KIND>
 __global__ void __attribute__((amdgpu_flat_work_group_size(kBwdThreads, kBwdThreads), amdgpu_waves_per_eu(2, 2)))
 attn_bwd_kernel(const BwdParams p) {
-    static_assert(!SPILL || KIND == KIND_DKDV, "only the dK/dV kernel forms whole tiles of dS");
     typedef BwdCfg<D, KIND> C;
-    typedef BwdScoreWave<T, D, KIND, SPILL> SW;
+    typedef BwdScoreWave<T, D, KIND> SW;
     typedef BwdOutputWave<T, D, KIND> OW;
     typedef typename VecOf<T>::v8 V8;
     typedef typename VecOf<T>::v4 V4;
@@ -464,20 +462,15 @@ attn_bwd_kernel(const BwdParams p) {
         asm volatile("" ::: "memory");
         w.scores_plain(sc0, sring);
         if (n_steps > 0 && need_mask(tile_at(0))) mask(sc0, tile_at(0));
-        // where this wavefront pair's dS tiles go: [local head][stream tile][4 blk + qw], this lane's 16 bytes
-        char* const ds_lane = SPILL ? p.ds + (int64_t)bhl * p.ds_head_bytes + ((int64_t)(4 * blk + qw) * 2 * kFragBytes + lane * 16) : nullptr;
-        const int64_t ds_row = (int64_t)p.n_kt_pad * 2 * kFragBytes;
-        int t_c = tile_at(0);           // tile whose scores are `cur`
         auto body = [&](int s, typename SW::Scores& cur, typename SW::Scores& nxt) {
-            __builtin_amdgcn_s_waitcnt(0xC07F);   // own hand-over stores of step s-1 done (lgkmcnt(0); the dS stores to memory are not waited for)
+            __builtin_amdgcn_s_waitcnt(0xC07F);   // own hand-over stores of step s-1 done (lgkmcnt(0))
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             if (s < n_steps) {
                 w.step(cur, nxt, sring + ((s + 1) % kRingS) * SP_BYTES, string + (s % kRingStats) * kFragBytes,
-                       lds0 + ph_base + (s & 1) * 4 * C::PH_BYTES, SPILL ? ds_lane + t_c * ds_row : nullptr);
+                       lds0 + ph_base + (s & 1) * 4 * C::PH_BYTES);
                 if (s + 1 < n_steps && need_mask(t_o)) mask(nxt, t_o);
             }
-            t_c = wrap_inc(t_c);
             t_o = wrap_inc(t_o);   // tile at sweep position s + 2
         };
         for (int s = 0; s <= n_steps; s += 2) {
@@ -549,6 +542,8 @@ attn_bwd_kernel(const BwdParams p) {
         }
     }
 }
+
+#include "attn_bwd_quad_gfx950.h"
 
 // ---------------------------------------------------------------------------------------------- head dim 256
 // At d = 256 the stationary rows of a wavefront are 128 registers and its accumulators up to 256, and a stream tile is
@@ -870,8 +865,13 @@ typedef void (*dq_from_ds_kernel_t)(const DqFromDsParams);
 
 // Keeping dS pays where the two products it saves are large next to the 4 bytes per score element it moves: head dim 128.
 inline bool spill_head_dim(int d) { return d == 128; }
+// head dim 128: the four-role dK/dV kernel, with or without keeping dS (the other head dims: attn_bwd_kernel<T, D, KIND_DKDV>)
 template <typename T>
-bwd_kernel_t pick_dkdv_spill(int d) { return d == 128 ? attn_bwd_kernel<T, 128, KIND_DKDV, true> : nullptr; }
+bwd_kernel_t pick_dkdv_quad(int d, bool keep_ds) {
+    if (d != 128) return nullptr;
+    return keep_ds ? attn_dkdv_quad_kernel<T, 128, true> : attn_dkdv_quad_kernel<T, 128, false>;
+}
+inline size_t dkdv_lds_bytes(int d, size_t two_role) { return d == 128 ? (size_t)QuadCfg<128>::LDS_BYTES : two_role; }
 template <typename T>
 dq_from_ds_kernel_t pick_dq_from_ds(int d) { return d == 128 ? attn_dq_from_ds_kernel<T, 128> : nullptr; }
 
@@ -997,6 +997,8 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
     const bool bf16 = d->dtype == COSMOS_ATTN_BF16;
     const bool wide = d->d == 256;
     bwd_kernel_t k_dkdv = bf16 ? pick_bwd<__bf16, KIND_DKDV>(d->d) : pick_bwd<_Float16, KIND_DKDV>(d->d);
+    if (bwd_kernel_t quad = bf16 ? pick_dkdv_quad<__bf16>(d->d, false) : pick_dkdv_quad<_Float16>(d->d, false)) k_dkdv = quad;
+    const size_t lds_dkdv = dkdv_lds_bytes(d->d, g.lds_dkdv);
     bwd_kernel_t k_dq = bf16 ? pick_bwd<__bf16, KIND_DQ>(d->d) : pick_bwd<_Float16, KIND_DQ>(d->d);
     if (!wide && (!k_dkdv || !k_dq)) return COSMOS_ATTN_UNSUPPORTED;
     char* ws = (char*)workspace;
@@ -1067,7 +1069,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
     };
     if (g.spill) {
         // dS kept: per group of heads, the dK/dV kernel (which writes the group's dS tiles), then the pass that turns them into dQ
-        bwd_kernel_t k_spill = bf16 ? pick_dkdv_spill<__bf16>(d->d) : pick_dkdv_spill<_Float16>(d->d);
+        bwd_kernel_t k_spill = bf16 ? pick_dkdv_quad<__bf16>(d->d, true) : pick_dkdv_quad<_Float16>(d->d, true);
         dq_from_ds_kernel_t k_ds = bf16 ? pick_dq_from_ds<__bf16>(d->d) : pick_dq_from_ds<_Float16>(d->d);
         if (!k_spill || !k_ds) return COSMOS_ATTN_UNSUPPORTED;
         const size_t lds_ds = (size_t)kDsRing * (kDqWaves * 2 * kFragBytes + 2 * g.ndb * kFragBytes);
@@ -1083,7 +1085,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
             const int heads = BH - bh0 < g.group ? BH - bh0 : g.group;
             const BwdGeom::Plan pl = heads == g.group ? g.dkdv : BwdGeom::plan(g.dkdv.n_blk, heads, g.n_q_tiles, d->causal != 0);
             bp.bh0 = bh0;
-            if (!launch(k_spill, g.lds_dkdv, pl, bp, true)) return COSMOS_ATTN_LAUNCH_FAILED;
+            if (!launch(k_spill, lds_dkdv, pl, bp, true)) return COSMOS_ATTN_LAUNCH_FAILED;
             qp.bh0 = bh0;
             hipLaunchKernelGGL(k_ds, dim3((unsigned)(qp.n_blk * heads)), dim3(kDqThreads), lds_ds, stream, qp);
         }
@@ -1091,7 +1093,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
     }
     {
         set_dkdv();
-        if (!launch(k_dkdv, g.lds_dkdv, g.dkdv, bp, true)) return COSMOS_ATTN_LAUNCH_FAILED;
+        if (!launch(k_dkdv, lds_dkdv, g.dkdv, bp, true)) return COSMOS_ATTN_LAUNCH_FAILED;
     }
     {   // dQ: stationary queries, streamed keys
         bp.st1 = d->q; bp.s1_sb = d->q_stride[0]; bp.s1_sh = d->q_stride[1]; bp.s1_sl = d->q_stride[2];
