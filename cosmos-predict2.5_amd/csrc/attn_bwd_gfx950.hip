@@ -714,7 +714,7 @@ __global__ void __launch_bounds__(256) bwd_combine_kernel(const BwdParams p, int
 // element; K^T comes from the L2).  A workgroup owns 256 queries, one 32-query tile per wavefront (8 wavefronts, two per
 // SIMD); per 32-key step a wavefront copies its own 2 KB dS tile and an eighth of the shared 32-key K^T part into an LDS
 // ring with direct-to-LDS loads kDsRing - 1 steps ahead, and accumulates dQ^T += K^T W with W = dS^T.
-// A dS tile lies in memory as the dK/dV kernel's score wavefront held it -- lane = key, eight queries per 16 bytes -- and is
+// A dS tile lies in memory in the 16-byte units the dK/dV kernel's wavefront held -- one key, eight queries -- and is
 // wanted with lane = query, eight keys per lane: the transposing LDS read (ds_read_b64_tr_b16) does that.  Within a
 // group of 16 lanes, lane i passes the address of 8 bytes (row i of a 16 x 4 matrix M of 16-bit values) and receives
 // M[i/4 + 4k][i%4], k = 0..3.  A row of M here is one key's dS for 4 consecutive queries, so lane (query, half hh) gets, for
@@ -793,11 +793,12 @@ attn_dq_from_ds_kernel(const DqFromDsParams p) {
     }
     // transposing read: byte offset, inside a dS tile, of the 8 bytes this lane passes for key chunk 0, read 0
     //   group g = lane / 16: queries 16 (g % 2) .. + 15, key half g / 2;  lane i of the group passes row r = i:
-    //   queries 16 (g%2) + 4 (r%4) .. + 3 of key 4 (g/2) + r/4  (+ 16 c + 8 t).  In the tile: fragment g%2 (queries 16 (g%2) ..),
-    //   lane index key + 32 (r%2), second 8 bytes of the lane's 16 when (r%4)/2.
+    //   queries 16 (g%2) + 4 (r%4) .. + 3 of key 4 (g/2) + r/4  (+ 16 c + 8 t).  In the tile the 16-byte unit (query half c' = g%2,
+    //   key, lane half hh' = r%2 of the wavefront that formed it) sits at slot 16 (key / 4) + 8 c' + 4 hh' + key % 4, and the lane
+    //   wants its second 8 bytes when (r%4)/2: the 32 lanes of a pass touch 256 consecutive bytes, every bank once.
     const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;   // LDS address of smem[0]
     const int g16 = lane >> 4, r16 = lane & 15;
-    const unsigned tr_off = (unsigned)((g16 & 1) * kFragBytes + (4 * (g16 >> 1) + (r16 >> 2) + 32 * (r16 & 1)) * 16 + 8 * ((r16 & 3) >> 1));
+    const unsigned tr_off = (unsigned)(256 * (g16 >> 1) + 128 * (g16 & 1) + 64 * (r16 & 1) + 16 * (r16 >> 2) + 8 * ((r16 & 3) >> 1));
 
     for (int s = 0; s < n_steps; ++s) {
         __builtin_amdgcn_s_waitcnt(WAIT_LOADS);
@@ -811,9 +812,9 @@ attn_dq_from_ds_kernel(const DqFromDsParams p) {
         const unsigned wt = lds0 + (unsigned)((s % kDsRing) * C::SLOT_BYTES + wave * C::W_BYTES) + tr_off;
         s16x4 t00, t01, t10, t11;
         asm volatile("ds_read_b64_tr_b16 %0, %4\n\t"
-                     "ds_read_b64_tr_b16 %1, %4 offset:128\n\t"
-                     "ds_read_b64_tr_b16 %2, %4 offset:256\n\t"
-                     "ds_read_b64_tr_b16 %3, %4 offset:384\n\t"
+                     "ds_read_b64_tr_b16 %1, %4 offset:512\n\t"
+                     "ds_read_b64_tr_b16 %2, %4 offset:1024\n\t"
+                     "ds_read_b64_tr_b16 %3, %4 offset:1536\n\t"
                      "s_waitcnt lgkmcnt(0)"
                      : "=&v"(t00), "=&v"(t01), "=&v"(t10), "=&v"(t11) : "v"(wt) : "memory");
         V8 wf[2];

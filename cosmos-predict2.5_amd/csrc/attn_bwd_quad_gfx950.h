@@ -230,7 +230,9 @@ attn_dkdv_quad_kernel(const BwdParams p) {
             }
         } else {
             // ---------------------------------------------------------------- S2
-            char* const ds_lane = SPILL ? p.ds + (int64_t)bhl * p.ds_head_bytes + ((int64_t)(4 * blk + 2 * grp) * 2 * kFragBytes + lane * 16) : nullptr;
+            // Inside a 2 KB tile the 16-byte unit (query half c', key, lane half hh) sits at slot 16 (key / 4) + 8 c' + 4 hh + key % 4: the
+            // order in which the transposing reads of attn_dq_from_ds_kernel touch 256 consecutive bytes per pass (no bank conflicts).
+            char* const ds_lane = SPILL ? p.ds + (int64_t)bhl * p.ds_head_bytes + ((int64_t)(4 * blk + 2 * grp) * 2 * kFragBytes + 16 * (16 * (j >> 2) + 4 * hh + (j & 3))) : nullptr;
             const int64_t ds_row = (int64_t)p.n_kt_pad * 2 * kFragBytes;
             int t_prev = tile_at(0);      // tile whose W the step forms (sweep position s - 1)
             // one step: MFMAs of dP(s) into xc (if CUR) interleaved with W(s-1) = U(s-1) * (dP(s-1) - D) from xp (if PREV)
@@ -288,9 +290,9 @@ attn_dkdv_quad_kernel(const BwdParams p) {
                     if (SPILL) {   // the two 32-key tiles of dS of this group: [stream tile][4 blk + 2 grp + hf], this lane's 2 x 16 bytes each
                         char* dst = ds_lane + t_prev * ds_row;
                         __builtin_nontemporal_store(wf[0][0], reinterpret_cast<V8*>(dst));
-                        __builtin_nontemporal_store(wf[0][1], reinterpret_cast<V8*>(dst + kFragBytes));
+                        __builtin_nontemporal_store(wf[0][1], reinterpret_cast<V8*>(dst + 128));
                         __builtin_nontemporal_store(wf[1][0], reinterpret_cast<V8*>(dst + 2 * kFragBytes));
-                        __builtin_nontemporal_store(wf[1][1], reinterpret_cast<V8*>(dst + 3 * kFragBytes));
+                        __builtin_nontemporal_store(wf[1][1], reinterpret_cast<V8*>(dst + 2 * kFragBytes + 128));
                     }
                 }
             };
