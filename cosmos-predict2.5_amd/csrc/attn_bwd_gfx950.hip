@@ -115,12 +115,21 @@ __global__ void __launch_bounds__(kPackThreads) bwd_stats_kernel(const StatsPara
 }
 
 // ---------------------------------------------------------------------------------------------- stream re-tiling
+// Order of the 16-byte units (row q of the tile, 16-channel chunk cK, half hK: 8 channels) inside a K-type section of the
+// query stream of attn_dkdv_quad_kernel, which reads the same units linearly (ds_read_b128, lane = row) and transposed
+// (ds_read_b64_tr_b16): both without bank conflicts in this order (attn_bwd_quad_gfx950.h).
+__host__ __device__ constexpr int quad_unit_slot(int q, int cK, int hK) {
+    return 16 * ((q >> 4) + 2 * hK + 4 * cK) + ((q & 3) + 4 * (((q >> 2) & 3) ^ (hK + 2 * (cK & 1))));
+}
+
 struct PackSrc { const uint16_t* ptr; int64_t sb, sh, sl; };
 struct PackBwdParams {
-    PackSrc a1, a2, c1, c2;      // c2.ptr may be null (no second V^T-type section)
+    PackSrc a1, a2, c1, c2;      // the K-type sections and the V^T-type sections (n_vt of them: 0, 1 or 2)
     const float2* stats;         // null: no statistics fragment
     uint4* out;
     int H, L, d, n_tiles, nc, ndb, tile_frags;
+    int n_vt;                    // number of V^T-type sections
+    int swz;                     // K-type sections in the unit order of attn_dkdv_quad_kernel (quad_unit_slot) instead of fragment by fragment
 };
 
 // grid (n_tiles, B*H); every 16-byte unit of a tile image is produced by one thread.
@@ -133,13 +142,16 @@ __global__ void __launch_bounds__(kPackThreads) pack_stream_kernel(const PackBwd
         int frag = u >> 6;
         const int l = u & 63, i = l & 31, hh = l >> 5;
         uint4 val = make_uint4(0u, 0u, 0u, 0u);
+        int where = u;           // 16-byte unit of the tile image this value goes to
         if (frag < ktype_frags) {
-            const PackSrc& s = frag < p.nc ? p.a1 : p.a2;
-            if (frag >= p.nc) frag -= p.nc;
+            const int sec = frag < p.nc ? 0 : 1;
+            const PackSrc& s = sec ? p.a2 : p.a1;
+            frag -= sec * p.nc;
             const int row = t * kRows + i;
             if (row < p.L)
                 val = *reinterpret_cast<const uint4*>(s.ptr + (int64_t)b * s.sb + (int64_t)h * s.sh + (int64_t)row * s.sl + 16 * frag + 8 * hh);
-        } else if (frag < ktype_frags + vt_frags * (p.c2.ptr ? 2 : 1)) {
+            if (p.swz) where = sec * p.nc * 64 + quad_unit_slot(i, frag, hh);
+        } else if (frag < ktype_frags + vt_frags * p.n_vt) {
             frag -= ktype_frags;
             const PackSrc& s = frag < vt_frags ? p.c1 : p.c2;
             if (frag >= vt_frags) frag -= vt_frags;
@@ -169,7 +181,7 @@ __global__ void __launch_bounds__(kPackThreads) pack_stream_kernel(const PackBwd
             val = make_uint4(__builtin_bit_cast(uint32_t, f[0]), __builtin_bit_cast(uint32_t, f[1]),
                              __builtin_bit_cast(uint32_t, f[2]), __builtin_bit_cast(uint32_t, f[3]));
         }
-        dst[u] = val;
+        dst[where] = val;
     }
 }
 
@@ -897,7 +909,8 @@ struct BwdGeom {
     size_t stats_bytes, q_img_bytes, k_img_bytes;
     explicit BwdGeom(const cosmos_attn_bwd_desc* d) {
         nc = d->d / 16; ndb = (d->d + 31) / 32;
-        q_tile_bytes = (size_t)(2 * nc + 4 * ndb + 1) * kFragBytes;
+        quad = d->d == 128;   // attn_dkdv_quad_kernel: one copy of the query stream ([Q | dO | statistics])
+        q_tile_bytes = (size_t)(quad ? 2 * nc + 1 : 2 * nc + 4 * ndb + 1) * kFragBytes;
         k_tile_bytes = (size_t)(2 * nc + 2 * ndb) * kFragBytes;
         lds_dkdv = (size_t)kRingS * 2 * nc * kFragBytes + (size_t)kRingO * 4 * ndb * kFragBytes + 2 * 4 * 4 * kFragBytes + kRingStats * kFragBytes;
         lds_dq = (size_t)kRingS * 2 * nc * kFragBytes + (size_t)kRingO * 2 * ndb * kFragBytes + 2 * 4 * 2 * kFragBytes;
@@ -938,6 +951,7 @@ struct BwdGeom {
         part_bytes = ((p1 > p2 ? p1 : p2) + 1023) / 1024 * 1024;     // the two kernels run one after the other
     }
     static constexpr int kDefaultDsMiB = 32 * 1024;
+    bool quad = false;
     bool spill = false;
     int group = 0, n_kt_pad = 0;        // heads per group; key tiles per query tile in the dS buffer
     size_t ds_head_bytes = 0, ds_bytes = 0;
@@ -1041,6 +1055,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
         PackBwdParams pp;
         pp.a1 = src_of(d->q, d->q_stride); pp.a2 = src_of(d->dout, d->dout_stride);
         pp.c1 = src_of(d->dout, d->dout_stride); pp.c2 = src_of(d->q, d->q_stride);
+        pp.n_vt = g.quad ? 0 : 2; pp.swz = g.quad ? 1 : 0;
         pp.stats = stats; pp.out = (uint4*)q_img;
         pp.H = d->H; pp.L = d->Lq; pp.d = d->d; pp.n_tiles = g.n_q_tiles; pp.nc = g.nc; pp.ndb = g.ndb;
         pp.tile_frags = (int)(g.q_tile_bytes / kFragBytes);
@@ -1050,6 +1065,7 @@ COSMOS_ATTN_API int cosmos_attn_bwd(const cosmos_attn_bwd_desc* d, void* workspa
         PackBwdParams pp;
         pp.a1 = src_of(d->k, d->k_stride); pp.a2 = src_of(d->v, d->v_stride);
         pp.c1 = src_of(d->k, d->k_stride); pp.c2 = PackSrc{nullptr, 0, 0, 0};
+        pp.n_vt = 1; pp.swz = 0;
         pp.stats = nullptr; pp.out = (uint4*)k_img;
         pp.H = d->H; pp.L = d->Lkv; pp.d = d->d; pp.n_tiles = g.n_k_tiles; pp.nc = g.spill ? 0 : g.nc; pp.ndb = g.ndb;
         pp.tile_frags = (int)(g.k_tile_bytes / kFragBytes);

@@ -18,31 +18,44 @@
 //
 // Pipeline, step s (tile = sweep position):   S1: MFMAs S(s+1) | U(s)      S2: MFMAs dP(s) | W(s-1)
 //                                             O1: tile s-1                 O2: tile s-2
-// LDS: rings of the four stream parts (Q 4 deep, dO 4, dO^T 3, Q^T 3: a part is fetched two to three steps before its one
-// step of use), U and W hand-over (two stages each), statistics ring (6).  All direct-to-LDS fills are issued by the O
-// wavefronts (nine 1 KB loads per wavefront and step); one s_barrier per step.
+//
+// One copy of the stream.  A tile is [Q | dO | LSE log2e, D]: 32 rows x 128 channels of each tensor as 16-byte units
+// (row q, 16-channel chunk cK, half hK: 8 channels).  S1 / S2 read them as MFMA A operands with ds_read_b128 (lane = row);
+// O1 / O2 need the transposed operands (lane = channel, 8 rows per lane) and get them from the SAME units with the
+// transposing read ds_read_b64_tr_b16 (within 16 lanes, lane i passes the address of 8 bytes -- row i of a 16 x 4 matrix M of
+// 16-bit values -- and receives M[i/4 + 4k][i%4], k = 0..3): no second, transposed copy of the tile in memory, in the fills
+// or in LDS.  For both kinds of read to be free of bank conflicts the units of a part are stored in the order
+//     slot(q, cK, hK) = 16 (q/16 + 2 hK + 4 cK) + (q%4 + 4 ((q/4)%4 XOR (hK + 2 (cK%2)))):
+// the 16 lanes of a ds_read_b128 pass (16 consecutive rows, one cK, one hK) and the 32 lanes of a transposing pass (4 rows x
+// 2 chunks x 2 halves, both 8-byte halves of each unit) touch 256 consecutive-bank bytes each.  pack_stream_kernel writes the
+// image in that order; the direct-to-LDS fills copy it linearly.
+// LDS: rings of the two stream parts (Q 7 deep: fetched three steps before S1 uses it, kept until O2 has used it three steps
+// later; dO 5 deep), U and W hand-over (two stages each), statistics ring (6).  All fills are issued by the O wavefronts (five
+// 1 KB loads per wavefront and step); one s_barrier per step.  The O wavefronts' LDS reads are written as asm (the compiler
+// would put vmcnt(0) in front of the transposing-read builtin: it takes it for an access that may alias the fills in flight),
+// with their own lgkmcnt waits, each tied to the registers it makes valid.
 
 template <int D>
 struct QuadCfg {
     static_assert(D == 128, "built for head dim 128");
     static constexpr int NC = D / 16, NDB = D / 32;
-    static constexpr int KP_BYTES = NC * kFragBytes;          // Q part, dO part of a tile (K-type fragments)
-    static constexpr int TP_BYTES = 2 * NDB * kFragBytes;     // dO^T part, Q^T part (V^T-type fragments)
-    static constexpr int Q_SRC = 0, DO_SRC = KP_BYTES, DOT_SRC = 2 * KP_BYTES, QT_SRC = 2 * KP_BYTES + TP_BYTES, ST_SRC = 2 * KP_BYTES + 2 * TP_BYTES;
-    static constexpr int TILE_BYTES = ST_SRC + kFragBytes;    // = the image of attn_bwd_kernel's query stream
-    static constexpr int RQ = 4, RDO = 4, RDOT = 3, RQT = 3, RST = 6;
+    static constexpr int KP_BYTES = NC * kFragBytes;          // Q part, dO part of a tile
+    static constexpr int Q_SRC = 0, DO_SRC = KP_BYTES, ST_SRC = 2 * KP_BYTES;
+    static constexpr int TILE_FRAGS = 2 * NC + 1;
+    static constexpr int TILE_BYTES = TILE_FRAGS * kFragBytes;
+    static constexpr int RQ = 7, RDO = 5, RST = 6;
     static constexpr int HO_BYTES = 4 * kFragBytes;           // hand-over of one group and stage: 64 keys x 32 queries, 16 bit
     static constexpr int Q_OFF = 0;
     static constexpr int DO_OFF = Q_OFF + RQ * KP_BYTES;
-    static constexpr int DOT_OFF = DO_OFF + RDO * KP_BYTES;
-    static constexpr int QT_OFF = DOT_OFF + RDOT * TP_BYTES;
-    static constexpr int U_OFF = QT_OFF + RQT * TP_BYTES;     // [2 stages][2 groups]
+    static constexpr int U_OFF = DO_OFF + RDO * KP_BYTES;     // [2 stages][2 groups]
     static constexpr int W_OFF = U_OFF + 4 * HO_BYTES;
     static constexpr int ST_OFF = W_OFF + 4 * HO_BYTES;
     static constexpr int LDS_BYTES = ST_OFF + RST * kFragBytes;
-    static constexpr int LOADS = 9;                           // per O wavefront and step: 2 fragments of each part + the statistics
-    static constexpr int IN_FLIGHT = 14;                      // at the top of a step: all but the newest 14 loads must have landed
+    static constexpr int LOADS = 5;                           // per O wavefront and step: 2 fragments of each part + the statistics
+    static constexpr int IN_FLIGHT = 2 * LOADS;               // at the top of a step: all but the loads of the last two steps must have landed
 };
+
+typedef short quad_s16x4 __attribute__((ext_vector_type(4)));
 
 template <typename T, int D, bool SPILL>
 __global__ void __attribute__((amdgpu_flat_work_group_size(kBwdThreads, kBwdThreads), amdgpu_waves_per_eu(2, 2)))
@@ -85,6 +98,9 @@ attn_dkdv_quad_kernel(const BwdParams p) {
         const_cast<char*>(p.stream) + (size_t)bh * p.n_tiles * C::TILE_BYTES, 0, p.n_tiles * C::TILE_BYTES, 0x00020000);
     const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
     auto frag = [&](const char* base, int f) { return *reinterpret_cast<const V8*>(base + f * kFragBytes + lane * 16); };
+    // A fragment cK of a stream part (lane = row j, half hh): byte offset of this lane's unit, for even / odd cK
+    const int a_off[2] = {16 * quad_unit_slot(j, 0, hh), 16 * quad_unit_slot(j, 1, hh) - kFragBytes};
+    auto afrag = [&](const char* part, int cK) { return *reinterpret_cast<const V8*>(part + cK * kFragBytes + a_off[cK & 1]); };
 
     // ---- fills (O wavefronts): this wavefront's two fragments of a part of tile t into ring slot u
     const int run = 2 * ow * kFragBytes;
@@ -96,12 +112,10 @@ attn_dkdv_quad_kernel(const BwdParams p) {
         lds_load<0>(rsrc, smem + C::ST_OFF + (u % C::RST) * kFragBytes, lane * 16, t * C::TILE_BYTES + C::ST_SRC);
     };
     auto fill_do = [&](int t, int u) { fill_part(C::DO_SRC, C::DO_OFF, C::KP_BYTES, C::RDO, t, u); };
-    auto fill_dot = [&](int t, int u) { fill_part(C::DOT_SRC, C::DOT_OFF, C::TP_BYTES, C::RDOT, t, u); };
-    auto fill_qt = [&](int t, int u) { fill_part(C::QT_SRC, C::QT_OFF, C::TP_BYTES, C::RQT, t, u); };
-    if (!s_role) {   // what steps -3, -2, -1 would have issued
-        fill_q(tile_at(0), 0); fill_do(tile_at(0), 0); fill_q(tile_at(1), 1);
-        fill_do(tile_at(1), 1); fill_q(tile_at(2), 2);
-        fill_dot(tile_at(0), 0); fill_do(tile_at(2), 2); fill_q(tile_at(3), 3);
+    if (!s_role) {   // what the steps before step 0 would have issued
+        fill_q(tile_at(0), 0);
+#pragma unroll
+        for (int u = 0; u < 3; ++u) { fill_do(tile_at(u), u); fill_q(tile_at(u + 1), u + 1); }
     }
 
     const unsigned u_base = C::U_OFF + grp * C::HO_BYTES, w_base = C::W_OFF + grp * C::HO_BYTES;   // + stage * 2 * HO_BYTES
@@ -152,7 +166,7 @@ attn_dkdv_quad_kernel(const BwdParams p) {
             if (n > 0) {
 #pragma unroll
                 for (int c = 0; c < NC; ++c) {
-                    const V8 fa = frag(smem + C::Q_OFF, c);
+                    const V8 fa = afrag(smem + C::Q_OFF, c);
                     x0[0] = mfma32(fa, breg[0][c], x0[0]);
                     x0[1] = mfma32(fa, breg[1][c], x0[1]);
                 }
@@ -160,24 +174,24 @@ attn_dkdv_quad_kernel(const BwdParams p) {
             }
             int t_next = tile_at(1);      // tile whose scores the step computes
             // one step: MFMAs of S(s+1) into xn (if NEXT) interleaved with U(s) from x (if CUR)
+            float l2v[16];
+            auto load_l2 = [&](const char* stats) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float4 a = *reinterpret_cast<const float4*>(stats + 64 * hh + 16 * i);
+                    l2v[4 * i] = a.x; l2v[4 * i + 1] = a.y; l2v[4 * i + 2] = a.z; l2v[4 * i + 3] = a.w;
+                }
+            };
             auto step = [&](auto NEXT, auto CUR, const f32x16* x, f32x16* xn, int s) {
                 constexpr bool next = decltype(NEXT)::value, cur = decltype(CUR)::value;
                 const char* qpart = smem + C::Q_OFF + ((s + 1) % C::RQ) * C::KP_BYTES;
-                const char* stats = smem + C::ST_OFF + (s % C::RST) * kFragBytes;
                 V8 uf[2][2];
                 V8 fa[NC];
-                float l2v[16];
                 if (next) {
 #pragma unroll
-                    for (int i = 0; i < PD; ++i) fa[i] = frag(qpart, i);
+                    for (int i = 0; i < PD; ++i) fa[i] = afrag(qpart, i);
                 }
-                if (cur) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float4 a = *reinterpret_cast<const float4*>(stats + 64 * hh + 16 * i);
-                        l2v[4 * i] = a.x; l2v[4 * i + 1] = a.y; l2v[4 * i + 2] = a.z; l2v[4 * i + 3] = a.w;
-                    }
-                }
+                if (cur) load_l2(smem + C::ST_OFF + (s % C::RST) * kFragBytes);
                 if (next) {
 #pragma unroll
                     for (int hf = 0; hf < 2; ++hf) {
@@ -188,7 +202,7 @@ attn_dkdv_quad_kernel(const BwdParams p) {
 #pragma unroll
                 for (int c = 0; c < NC; ++c) {
                     SCHED_FENCE();
-                    if (next && c + PD < NC) fa[c + PD] = frag(qpart, c + PD);
+                    if (next && c + PD < NC) fa[c + PD] = afrag(qpart, c + PD);
                     SCHED_FENCE();
 #pragma unroll
                     for (int hf = 0; hf < 2; ++hf) {
@@ -236,26 +250,28 @@ attn_dkdv_quad_kernel(const BwdParams p) {
             const int64_t ds_row = (int64_t)p.n_kt_pad * 2 * kFragBytes;
             int t_prev = tile_at(0);      // tile whose W the step forms (sweep position s - 1)
             // one step: MFMAs of dP(s) into xc (if CUR) interleaved with W(s-1) = U(s-1) * (dP(s-1) - D) from xp (if PREV)
+            float ddv[16];
+            auto load_dd = [&](const char* stats) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float4 a = *reinterpret_cast<const float4*>(stats + 128 + 64 * hh + 16 * i);
+                    ddv[4 * i] = a.x; ddv[4 * i + 1] = a.y; ddv[4 * i + 2] = a.z; ddv[4 * i + 3] = a.w;
+                }
+            };
             auto step = [&](auto CUR, auto PREV, f32x16* xc, const f32x16* xp, int s) {
                 constexpr bool cur = decltype(CUR)::value, prev = decltype(PREV)::value;
                 const char* dopart = smem + C::DO_OFF + (s % C::RDO) * C::KP_BYTES;
-                const char* stats = smem + C::ST_OFF + ((s + C::RST - 1) % C::RST) * kFragBytes;
                 const char* uin = smem + u_base + ((s + 1) & 1) * 2 * C::HO_BYTES;
                 V8 ui[2][2], wf[2][2];
                 V8 fb[NC];
-                float ddv[16];
                 if (prev) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) ui[i >> 1][i & 1] = frag(uin, i);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float4 a = *reinterpret_cast<const float4*>(stats + 128 + 64 * hh + 16 * i);
-                        ddv[4 * i] = a.x; ddv[4 * i + 1] = a.y; ddv[4 * i + 2] = a.z; ddv[4 * i + 3] = a.w;
-                    }
+                    load_dd(smem + C::ST_OFF + ((s + C::RST - 1) % C::RST) * kFragBytes);
                 }
                 if (cur) {
 #pragma unroll
-                    for (int i = 0; i < PD; ++i) fb[i] = frag(dopart, i);
+                    for (int i = 0; i < PD; ++i) fb[i] = afrag(dopart, i);
 #pragma unroll
                     for (int hf = 0; hf < 2; ++hf) {
 #pragma unroll
@@ -265,7 +281,7 @@ attn_dkdv_quad_kernel(const BwdParams p) {
 #pragma unroll
                 for (int c = 0; c < NC; ++c) {
                     SCHED_FENCE();
-                    if (cur && c + PD < NC) fb[c + PD] = frag(dopart, c + PD);
+                    if (cur && c + PD < NC) fb[c + PD] = afrag(dopart, c + PD);
                     SCHED_FENCE();
 #pragma unroll
                     for (int hf = 0; hf < 2; ++hf) {
@@ -325,44 +341,65 @@ attn_dkdv_quad_kernel(const BwdParams p) {
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        int t_qt = tile_at(0), t_dot = tile_at(1), t_do = tile_at(3), t_q = tile_at(4);
+        int t_do = tile_at(3), t_q = tile_at(4);
         const int lag = second ? 2 : 1;                       // O1 accumulates tile s-1, O2 tile s-2
+        // Transposing reads.  Lane (group g = lane / 16, r = lane % 16) is channel 16 (g%2) + r of a 32-channel block and key-index
+        // half g/2 of the MFMA A operand; as a supplier of addresses it passes, for fragment (db, c) and read t, the 8 bytes of row
+        // q = 16 c + 8 t + 4 (g/2) + r/4, channels 32 db + 16 (g%2) + 4 (r%4) .. + 3: unit (q, cK = 2 db + g%2, hK = (r%4)/2), its
+        // second half when r is odd.  Byte offset in the part = 256 c + 2048 db + tr_off[t].
+        const int g16 = lane >> 4, r16 = lane & 15, hK = (r16 & 3) >> 1;
+        unsigned tr_off[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+            tr_off[t] = (unsigned)(512 * hK + 1024 * (g16 & 1) + 16 * (r16 >> 2) + 64 * ((2 * t + (g16 >> 1)) ^ (hK + 2 * (g16 & 1))) + 8 * (r16 & 1));
+// one MFMA group's A operand: fragment (db, c) = two transposing reads (t = 0, 1); IMM = 256 c + 2048 db
+#define QUAD_TR_PAIR(g) asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%4\n\tds_read_b64_tr_b16 %1, %3 offset:%4" \
+                                     : "=&v"(lo[g]), "=&v"(hi[g]) : "v"(ta0), "v"(ta1), "n"(256 * ((g) / NDB) + 2048 * ((g) % NDB)) : "memory")
+// wait until at most N of this wavefront's LDS reads are outstanding; ties the registers the wait makes valid
+#define QUAD_WAIT(N, g) asm volatile("s_waitcnt lgkmcnt(" #N ")" : "+v"(lo[g]), "+v"(hi[g]), "+v"(bf[0][0]), "+v"(bf[0][1]), "+v"(bf[1][0]), "+v"(bf[1][1]) :: "memory")
+#define QUAD_GROUP(g) do { \
+            const V8 fa = __builtin_shufflevector(__builtin_bit_cast(V4, lo[g]), __builtin_bit_cast(V4, hi[g]), 0, 1, 2, 3, 4, 5, 6, 7); \
+            acc[0][(g) % NDB] = mfma32(fa, bf[0][(g) / NDB], acc[0][(g) % NDB]); \
+            acc[1][(g) % NDB] = mfma32(fa, bf[1][(g) / NDB], acc[1][(g) % NDB]); } while (0)
+        static_assert(NB == 8, "the MFMA groups below are written out for head dim 128");
         for (int s = 0; s <= n + 1; ++s) {
             __builtin_amdgcn_s_waitcnt(WAIT_FILLS);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             const int u = s - lag;                             // sweep position accumulated in this step
             const bool active = u >= 0 && u < n;
-            const char* apart = second ? smem + C::QT_OFF + ((u + C::RQT) % C::RQT) * C::TP_BYTES
-                                       : smem + C::DOT_OFF + ((u + C::RDOT) % C::RDOT) * C::TP_BYTES;
+            // O1: dO part of tile u; O2: Q part of tile u
+            const unsigned part = lds0 + (second ? C::Q_OFF + ((u + C::RQ) % C::RQ) * C::KP_BYTES : C::DO_OFF + ((u + C::RDO) % C::RDO) * C::KP_BYTES);
+            const unsigned ta0 = part + tr_off[0], ta1 = part + tr_off[1];
             // U(u) was written in step u (stage u & 1), W(u) in step u + 1 (stage u & 1 as well)
-            const char* hin = smem + (second ? w_base : u_base) + (u & 1) * 2 * C::HO_BYTES;
+            const unsigned hin = lds0 + (second ? w_base : u_base) + (u & 1) * 2 * C::HO_BYTES + 16 * lane;
             V8 bf[2][2];
-            V8 fa[NB];
+            quad_s16x4 lo[NB], hi[NB];
             if (active) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) bf[i >> 1][i & 1] = frag(hin, i);
-#pragma unroll
-                for (int i = 0; i < PDO; ++i) fa[i] = frag(apart, 2 * (i % NDB) + i / NDB);
+                asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:1024\n\tds_read_b128 %2, %4 offset:2048\n\tds_read_b128 %3, %4 offset:3072"
+                             : "=&v"(bf[0][0]), "=&v"(bf[0][1]), "=&v"(bf[1][0]), "=&v"(bf[1][1]) : "v"(hin) : "memory");
+                QUAD_TR_PAIR(0); QUAD_TR_PAIR(1);
             }
             SCHED_FENCE();
-            // Q^T(s), dO^T(s+1), dO(s+3), Q(s+4) + statistics(s+4): into slots that were read for the last time in step s-1 or before
-            fill_qt(t_qt, s); fill_dot(t_dot, s + 1); fill_do(t_do, s + 3); fill_q(t_q, s + 4);
-            t_qt = wrap_inc(t_qt); t_dot = wrap_inc(t_dot); t_do = wrap_inc(t_do); t_q = wrap_inc(t_q);
+            // dO(s+3), Q(s+4) + statistics(s+4): into slots that were read for the last time in step s-1 or before
+            fill_do(t_do, s + 3); fill_q(t_q, s + 4);
+            t_do = wrap_inc(t_do); t_q = wrap_inc(t_q);
             SCHED_FENCE();
             if (active) {
-#pragma unroll
-                for (int g = 0; g < NB; ++g) {
-                    const int c = g / NDB, db = g % NDB;
-                    SCHED_FENCE();
-                    if (g + PDO < NB) fa[g + PDO] = frag(apart, 2 * ((g + PDO) % NDB) + (g + PDO) / NDB);
-                    SCHED_FENCE();
-                    acc[0][db] = mfma32(fa[g], bf[0][c], acc[0][db]);
-                    acc[1][db] = mfma32(fa[g], bf[1][c], acc[1][db]);
-                }
+                QUAD_TR_PAIR(2); QUAD_WAIT(4, 0); QUAD_GROUP(0);
+                QUAD_TR_PAIR(3); QUAD_WAIT(4, 1); QUAD_GROUP(1);
+                QUAD_TR_PAIR(4); QUAD_WAIT(4, 2); QUAD_GROUP(2);
+                QUAD_TR_PAIR(5); QUAD_WAIT(4, 3); QUAD_GROUP(3);
+                QUAD_TR_PAIR(6); QUAD_WAIT(4, 4); QUAD_GROUP(4);
+                QUAD_TR_PAIR(7); QUAD_WAIT(4, 5); QUAD_GROUP(5);
+                QUAD_WAIT(2, 6); QUAD_GROUP(6);
+                QUAD_WAIT(0, 7); QUAD_GROUP(7);
             }
             SCHED_FENCE();
         }
+#undef QUAD_TR_PAIR
+#undef QUAD_WAIT
+#undef QUAD_GROUP
         __builtin_amdgcn_s_waitcnt(0x0F70);   // drain the (unused) trailing fills before the LDS is released
         // ---- epilogue: dV = dV^T (O1), dK = s dK^T (O2)
         const float sc = second ? p.sm_scale : 1.0f;
