@@ -41,7 +41,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c2": ((2 * 1.770e6 + 1.997e5) * 1024, "profiles/attn_fwd_sym_kernel_bf16_d128_workload_c2.txt"),
     "c5": ((2 * 326847 + 603763) * 1024, "profiles/attn_qstream_kernel_bf16_d128_workload_c5.txt"),
     # 8 groups of 2 heads: dK/dV kernel (FETCH 3.22954e6, WRITE 2.7991e7: the dS tiles) + dQ-from-dS pass (FETCH 1.45919e7, WRITE 4.2262e4)
-    "c3b": (8 * (2 * (3.22954e6 + 1.45919e7) + 2.7991e7 + 4.2262e4) * 1024, "profiles/attn_bwd_kernel_bf16_d128_workload_c3b.txt"),
+    "c3b": (8 * (2 * (1.23294e6 + 1.46726e7) + 2.7991e7 + 4.22606e4) * 1024, "profiles/attn_bwd_kernel_bf16_d128_workload_c3b.txt"),
 }
 _NO_TRAFFIC = (None, None)
 
@@ -190,7 +190,7 @@ def bench_backward(args, pkg, dev, desc_txt, B, H, Lq, Lkv, d, steps, warmup):
                    "executed_matmuls": 5, "pct_of_bf16_mfma_peak": 100.0 * flops / sec / 1e12 / PEAK_BF16_TFLOPS},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["c3b"][0], "traffic_source": MEASURED_TRAFFIC_BYTES["c3b"][1],
-                     "kernel": "cosmos_attn_bwd (per group of heads: attn_bwd_kernel dK/dV keeping dS, attn_dq_from_ds_kernel; 3 small launches)", "kernel_ms_avg": avg, "kernel_ms_min": min(ms)},
+                     "kernel": "cosmos_attn_bwd (per group of heads: attn_dkdv_quad_kernel keeping dS, attn_dq_from_ds_kernel; 3 small launches)", "kernel_ms_avg": avg, "kernel_ms_min": min(ms)},
     }
     return result
 

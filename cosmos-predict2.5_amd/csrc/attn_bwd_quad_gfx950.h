@@ -1,8 +1,8 @@
 // dK/dV kernel of the backward for head dim 128, four wavefront roles ("quad").  Included inside the anonymous namespace of
 // attn_bwd_gfx950.hip (uses BwdParams, kRows, kBlock, kBwdThreads, kBwdSweepStagger and attn_common_gfx950.h).
 //
-// Same mathematics and stream as attn_bwd_kernel<T, D, KIND_DKDV> (a workgroup owns 128 keys and streams 32-query tiles
-// [Q | dO | dO^T | Q^T | LSE log2e, D]), other division of labour.  There every MFMA takes a fresh 1 KB A fragment from LDS
+// Same mathematics as attn_bwd_kernel<T, D, KIND_DKDV> (a workgroup owns 128 keys and streams 32-query tiles, there
+// [Q | dO | dO^T | Q^T | LSE log2e, D]), other division of labour and a stream half the size.  There every MFMA takes a fresh 1 KB A fragment from LDS
 // and the four wavefront pairs of a workgroup each read the whole stream tile: 1.13 KB of LDS operand per MFMA.  Here a group of
 // four wavefronts serves 64 keys, so that every stream fragment feeds two MFMAs, and each wavefront has one job:
 //   S1  S = Q k^T for its 64 keys (K rows are register-resident B operands), U = P = exp2(S c - LSE') rounded to 16 bit,
