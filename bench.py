@@ -37,7 +37,7 @@ PEAK_BF16_TFLOPS = 256 * 4096 * 2.4e9 / 1e12
 # number ("traffic_source").  A workload without a counter run reports null.
 MEASURED_TRAFFIC_BYTES = {
     "c3": ((2 * 2.633e7 + 710537) * 1024, "profiles/attn_fwd_jvp_kernel_bf16_d128_workload_c3.txt"),
-    "nr": ((2 * 359158.94 + 675840.03) * 1024, "profiles/norm_rope_kernel_bf16_d128_workload_nr.txt"),
+    "nr": ((2 * 359157 + 676527) * 1024, "profiles/norm_rope_kernel_bf16_d128_workload_nr.txt"),
     "c2": ((2 * 1.770e6 + 1.997e5) * 1024, "profiles/attn_fwd_sym_kernel_bf16_d128_workload_c2.txt"),
     "c5": ((2 * 326847 + 603763) * 1024, "profiles/attn_qstream_kernel_bf16_d128_workload_c5.txt"),
     # 8 groups of 2 heads: dK/dV kernel (FETCH 3.22954e6, WRITE 2.7991e7: the dS tiles) + dQ-from-dS pass (FETCH 1.45919e7, WRITE 4.2262e4)

@@ -78,9 +78,9 @@ struct LoadJob {
     int k_src, v_src;        // byte offsets of this wavefront's runs in the packed buffer
     char *k_dst, *v_dst;     // LDS destinations of the runs
 };
-template <int IMM>
+template <int IMM, int AUX = 0>   // AUX: cache policy bits of the instruction (2 = non-temporal)
 __device__ __forceinline__ void lds_load(__amdgpu_buffer_rsrc_t rsrc, char* dst, int lane_off, int src) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane_off, src, IMM, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane_off, src, IMM, AUX);
 }
 template <int LOADS>
 __device__ __forceinline__ void issue_part(__amdgpu_buffer_rsrc_t rsrc, char* dst, int lane_off, int src) {

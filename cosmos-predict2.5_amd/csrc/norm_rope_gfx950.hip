@@ -21,6 +21,22 @@
 #include "cosmos_attn_hip.h"
 
 namespace {
+// The tensors of these kernels are touched once: loads and stores that do not displace anything in the caches.
+typedef unsigned nr_u32x2 __attribute__((ext_vector_type(2)));
+#ifndef NR_PLAIN
+__device__ __forceinline__ uint2 stream_load(const uint16_t* p) {
+    const nr_u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const nr_u32x2*>(p));
+    return make_uint2(v[0], v[1]);
+}
+__device__ __forceinline__ void stream_store(uint16_t* p, uint2 v) {
+    nr_u32x2 w; w[0] = v.x; w[1] = v.y;
+    __builtin_nontemporal_store(w, reinterpret_cast<nr_u32x2*>(p));
+}
+#else
+__device__ __forceinline__ uint2 stream_load(const uint16_t* p) { return *reinterpret_cast<const uint2*>(p); }
+__device__ __forceinline__ void stream_store(uint16_t* p, uint2 v) { *reinterpret_cast<uint2*>(p) = v; }
+#endif
+
 
 constexpr int kThreads = 256;
 
@@ -150,11 +166,11 @@ __global__ void __launch_bounds__(kThreads) norm_rope_kernel(const NormRopeParam
 #pragma unroll
         for (int i = 0; i < HS; ++i) {
             const int64_t o = (hb + i < n_heads ? hb + i : 0) * p.x_sh;
-            xlo[i] = *reinterpret_cast<const uint2*>(xp + o);
-            xhi[i] = *reinterpret_cast<const uint2*>(xp + o + D / 2);
+            xlo[i] = stream_load(xp + o);
+            xhi[i] = stream_load(xp + o + D / 2);
             if (TANGENT) {
-                dlo[i] = *reinterpret_cast<const uint2*>(txp + o);
-                dhi[i] = *reinterpret_cast<const uint2*>(txp + o + D / 2);
+                dlo[i] = stream_load(txp + o);
+                dhi[i] = stream_load(txp + o + D / 2);
             }
         }
 #pragma unroll
@@ -197,11 +213,11 @@ __global__ void __launch_bounds__(kThreads) norm_rope_kernel(const NormRopeParam
             }
             if (hb + hh < n_heads) {
                 const int64_t o = (hb + hh) * p.y_sh;
-                *reinterpret_cast<uint2*>(yp + o) = pack4<BF16>(y);
-                *reinterpret_cast<uint2*>(yp + o + D / 2) = pack4<BF16>(y + 4);
+                stream_store(yp + o, pack4<BF16>(y));
+                stream_store(yp + o + D / 2, pack4<BF16>(y + 4));
                 if (TANGENT) {
-                    *reinterpret_cast<uint2*>(typ + o) = pack4<BF16>(dy);
-                    *reinterpret_cast<uint2*>(typ + o + D / 2) = pack4<BF16>(dy + 4);
+                    stream_store(typ + o, pack4<BF16>(dy));
+                    stream_store(typ + o + D / 2, pack4<BF16>(dy + 4));
                 }
             }
         }
@@ -288,10 +304,10 @@ __global__ void __launch_bounds__(kThreads) norm_rope_bwd_kernel(const NormRopeB
 #pragma unroll
         for (int i = 0; i < HS; ++i) {
             const int hsel = hb + i < n_heads ? hb + i : 0;   // surplus slots re-read the first head, store nothing
-            xlo[i] = *reinterpret_cast<const uint2*>(xp + hsel * p.x_sh);
-            xhi[i] = *reinterpret_cast<const uint2*>(xp + hsel * p.x_sh + D / 2);
-            glo[i] = *reinterpret_cast<const uint2*>(gp + hsel * p.g_sh);
-            ghi[i] = *reinterpret_cast<const uint2*>(gp + hsel * p.g_sh + D / 2);
+            xlo[i] = stream_load(xp + hsel * p.x_sh);
+            xhi[i] = stream_load(xp + hsel * p.x_sh + D / 2);
+            glo[i] = stream_load(gp + hsel * p.g_sh);
+            ghi[i] = stream_load(gp + hsel * p.g_sh + D / 2);
         }
 #pragma unroll
         for (int hh = 0; hh < HS; ++hh) {
@@ -325,8 +341,8 @@ __global__ void __launch_bounds__(kThreads) norm_rope_bwd_kernel(const NormRopeB
 #pragma unroll
                 for (int i = 0; i < 8; ++i) wacc[i] += dn[i] * x[i] * r;
                 uint16_t* o = op + (int64_t)(hb + hh) * p.o_sh;
-                *reinterpret_cast<uint2*>(o) = pack4<BF16>(dx);
-                *reinterpret_cast<uint2*>(o + D / 2) = pack4<BF16>(dx + 4);
+                stream_store(o, pack4<BF16>(dx));
+                stream_store(o + D / 2, pack4<BF16>(dx + 4));
             }
         }
     }
