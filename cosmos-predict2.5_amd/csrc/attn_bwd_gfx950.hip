@@ -731,9 +731,7 @@ __global__ void __launch_bounds__(256) bwd_combine_kernel(const BwdParams p, int
 // group of 16 lanes, lane i passes the address of 8 bytes (row i of a 16 x 4 matrix M of 16-bit values) and receives
 // M[i/4 + 4k][i%4], k = 0..3.  A row of M here is one key's dS for 4 consecutive queries, so lane (query, half hh) gets, for
 // key chunk c and read t, the keys 16 c + 8 t + 4 hh + k -- the order in which a V^T-type fragment of K^T holds them.
-#ifndef DQ_DS_AUX
-#define DQ_DS_AUX 2
-#endif
+constexpr int kDsLoadPolicy = 2;     // cache policy bits of the dS loads: non-temporal (each tile is read once; 4 % faster than plain loads)
 constexpr int kDsRing = 6;            // steps of dS / K^T in flight per workgroup
 constexpr int kDqWaves = 8;           // query tiles per workgroup
 constexpr int kDqThreads = 64 * kDqWaves;
@@ -771,7 +769,6 @@ attn_dq_from_ds_kernel(const DqFromDsParams p) {
     // vmcnt(n): the loads of the newest kDsRing - 2 steps may still be in flight
     constexpr int IN_FLIGHT = C::LOADS * (kDsRing - 2);
     constexpr int WAIT_LOADS = (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14) | 0x0F70;
-    constexpr int WAIT_PAIR = (2 * C::LOADS) | 0x0F70;   // all but the loads of the newest pair of steps
 
     const int blk = blockIdx.x % p.n_blk, bhl = blockIdx.x / p.n_blk, bh = p.bh0 + bhl, b = bh / p.H, h = bh % p.H;
     const int lane = threadIdx.x & 63;
@@ -795,17 +792,12 @@ attn_dq_from_ds_kernel(const DqFromDsParams p) {
     auto issue = [&](int u) {                      // loads of sweep position u (clamped: positions past the end repeat the last tile, unused)
         const int t = __builtin_amdgcn_readfirstlane(u < n_steps ? u : n_steps - 1);
         char* slot = smem + (u % kDsRing) * C::SLOT_BYTES;
-        lds_load<0, DQ_DS_AUX>(rs_w, slot + wave * C::W_BYTES, lane * 16, t * C::W_BYTES);
-        lds_load<kFragBytes, DQ_DS_AUX>(rs_w, slot + wave * C::W_BYTES, lane * 16, t * C::W_BYTES);
+        lds_load<0, kDsLoadPolicy>(rs_w, slot + wave * C::W_BYTES, lane * 16, t * C::W_BYTES);
+        lds_load<kFragBytes, kDsLoadPolicy>(rs_w, slot + wave * C::W_BYTES, lane * 16, t * C::W_BYTES);
         lds_load<0>(rs_k, slot + kDqWaves * C::W_BYTES + kfrag * kFragBytes, lane * 16, t * C::KT_BYTES + kfrag * kFragBytes);
     };
-#ifdef DQ_PAIR
-#pragma unroll
-    for (int u = 0; u < 4; ++u) issue(u);
-#else
 #pragma unroll
     for (int u = 0; u < kDsRing - 1; ++u) issue(u);
-#endif
 
     f32x16 acc[NDB];
 #pragma unroll
@@ -858,17 +850,6 @@ attn_dq_from_ds_kernel(const DqFromDsParams p) {
                 acc[db] = mfma32(*reinterpret_cast<const V8*>(kt + (2 * db + c) * kFragBytes), wf[c], acc[db]);
         }
     };
-#ifdef DQ_PAIR
-    // two steps per barrier: the loads of a pair of steps are issued together (4 KB of dS per wavefront in one go)
-    for (int s = 0; s < n_steps; s += 2) {
-        __builtin_amdgcn_s_waitcnt(WAIT_PAIR);
-        __builtin_amdgcn_s_barrier();          // everybody's loads of steps s, s + 1 have landed, everybody is done reading steps s - 2, s - 1
-        asm volatile("" ::: "memory");
-        issue(s + 4); issue(s + 5);            // into the slots of steps s - 2, s - 1
-        step(s);
-        if (s + 1 < n_steps) step(s + 1);
-    }
-#else
     for (int s = 0; s < n_steps; ++s) {
         __builtin_amdgcn_s_waitcnt(WAIT_LOADS);
         __builtin_amdgcn_s_barrier();          // everybody's loads of step s have landed, everybody is done reading step s - 1
@@ -876,7 +857,6 @@ attn_dq_from_ds_kernel(const DqFromDsParams p) {
         issue(s + kDsRing - 1);                // into the slot of step s - 1
         step(s);
     }
-#endif
     __builtin_amdgcn_s_waitcnt(0x0F70);        // drain the trailing loads before the LDS is released
     if (live_tile && row < p.Lq) {
         T* o1 = reinterpret_cast<T*>(p.dq) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)row * p.o_sl;
