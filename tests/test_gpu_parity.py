@@ -56,6 +56,30 @@ def run_case(pkg, oracle, gpu, shape_q, shape_kv=None, dv=None, causal=False, sm
     return o, to, lse
 
 
+# ------------------------------------------------------------------ head dims 128 / 128, tangents on k and v, more than 2048 keys
+# (past what the query-streaming kernel takes: ragged tails, causal, key padding and key-range splits at that length)
+@pytest.mark.parametrize("Lq,Lkv", [(300, 2081), (128, 2112), (517, 4000), (1, 2049), (33, 3000)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_long_key_sequences_full_tangents(pkg, oracle, gpu, Lq, Lkv, dtype):
+    run_case(pkg, oracle, gpu, (1, 2, Lq, 128), (1, 2, Lkv, 128), seed=Lq + Lkv, dtype=dtype)
+
+
+@pytest.mark.parametrize("L", [2049, 2200, 2304])
+def test_long_key_sequences_causal(pkg, oracle, gpu, L):
+    run_case(pkg, oracle, gpu, (1, 2, L, 128), causal=True, seed=L)
+
+
+@pytest.mark.parametrize("lens", [[2100, 2600], [1, 2590], [2561, 33]])
+def test_long_key_sequences_key_padding(pkg, oracle, gpu, lens):
+    run_case(pkg, oracle, gpu, (2, 2, 200, 128), (2, 2, 2600, 128), key_lens=lens, seed=lens[0])
+
+
+def test_long_key_sequences_key_range_split_and_rms_normed_inputs(pkg, oracle, gpu):
+    # 4 (query block, head) pairs on 256 compute units: every pair is cut into 16 key ranges and merged
+    run_case(pkg, oracle, gpu, (1, 2, 256, 128), (1, 2, 4096, 128), seed=5, rms=True)
+    run_case(pkg, oracle, gpu, (1, 3, 200, 128), (1, 3, 2500, 128), seed=6, tangent_std=1.0)
+
+
 # ------------------------------------------------------------------ small and ragged shapes
 def test_smallest(pkg, oracle, gpu):
     run_case(pkg, oracle, gpu, (1, 1, 64, 128))
