@@ -41,7 +41,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c2": ((2 * 1.770e6 + 1.997e5) * 1024, "profiles/attn_fwd_sym_kernel_bf16_d128_workload_c2.txt"),
     "c5": ((2 * 326847 + 603763) * 1024, "profiles/attn_qstream_kernel_bf16_d128_workload_c5.txt"),
     # 8 groups of 2 heads: dK/dV kernel (FETCH 3.22954e6, WRITE 2.7991e7: the dS tiles) + dQ-from-dS pass (FETCH 1.45919e7, WRITE 4.2262e4)
-    "c3b": (8 * (2 * (1.23294e6 + 1.46726e7) + 2.7991e7 + 4.22606e4) * 1024, "profiles/attn_bwd_kernel_bf16_d128_workload_c3b.txt"),
+    "c3b": (8 * (2 * (1.23173e6 + 1.42848e7) + 2.7991e7 + 4.22565e4) * 1024, "profiles/attn_bwd_kernel_bf16_d128_workload_c3b.txt"),
 }
 _NO_TRAFFIC = (None, None)
 
